@@ -1,0 +1,483 @@
+// Dense L1 attention for gfx950 (MI355X): A[b,s,t,h] = -1/sqrt(W) * sum_w |q[b,t,h,w] - k[b,s,h,w]|
+// and its backward.  Replaces the kernels and launchers of the reference's
+// cuda/l1attn_cuda_kernel.cu:27-685 and the dispatch in cuda/l1attn_cuda_drv.cpp:42-104.
+//
+// The op is a non-contraction (|a-b| does not factor), so it runs on the fp32 VALU, not on MFMA.
+//
+// Forward (fp32 fast path): one wavefront per head, one lane per dst token t.  A lane keeps its
+// q row in registers; the k row of the current src token is wave-uniform and is read through the
+// scalar cache into SGPRs, so the inner loop is two VALU instructions per pair-element
+// (v_sub, v_add |x|) with no LDS or vector-memory traffic.  The workgroup (all heads of a 64-token
+// dst tile) transposes each finished src row through LDS and stores [t-tile x H] contiguous runs.
+//
+// Backward (fp32 fast path): one lane per (h,w) column, a workgroup per 32-token dst tile looping
+// over all src tokens.  q values and dq accumulators live in registers, the dA tile is staged
+// through LDS in [s][h][t] order so that a lane reads its head's four consecutive dA values with
+// one broadcast ds_read_b128.  Per pair-element: v_sub, v_med3 (sign with sign(0)=0), two v_fma.
+// dq is complete when the loop ends; dk is written as one partial per dst tile and summed in
+// tile order by a second kernel, so the result is bitwise reproducible (no atomics).
+//
+// Generic kernels (any shape, float or double, exact comparisons) cover everything else.
+#include "common.h"
+#include <math.h>
+#include <algorithm>
+
+namespace {
+
+constexpr int WAVE = 64;
+
+// ------------------------------------------------------------------------------------------
+// generic kernels
+// ------------------------------------------------------------------------------------------
+
+template <typename T>
+__device__ __forceinline__ T sgn_exact(T x) { return (T)((x > (T)0) - (x < (T)0)); }
+
+template <typename T>
+__device__ __forceinline__ T abs_t(T x) { return x < (T)0 ? -x : x; }
+
+// one thread per (t,h); blockIdx.y strides over (b,s)
+template <typename T>
+__global__ __launch_bounds__(256) void dense_fwd_generic(const T* __restrict__ q, const T* __restrict__ k,
+                                                           T* __restrict__ attn, int64_t B, int64_t Tn,
+                                                           int64_t H, int64_t W, T scale)
+{
+	int64_t th = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (th >= Tn * H) return;
+	int64_t h = th % H;
+	for (int64_t bs = blockIdx.y; bs < B * Tn; bs += gridDim.y) {
+		int64_t b = bs / Tn;
+		const T* qp = q + (b * Tn * H + th) * W;
+		const T* kp = k + (bs * H + h) * W;
+		T f = 0;
+		for (int64_t w = 0; w < W; w++) f += abs_t(qp[w] - kp[w]);
+		attn[bs * Tn * H + th] = f * scale;
+	}
+}
+
+// one thread per dq element, src tokens summed in ascending order
+template <typename T>
+__global__ __launch_bounds__(256) void dense_bwd_generic_dq(const T* __restrict__ dA, const T* __restrict__ q,
+                                                              const T* __restrict__ k, T* __restrict__ dq,
+                                                              int64_t B, int64_t Tn, int64_t H, int64_t W, T scale)
+{
+	int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= B * Tn * H * W) return;
+	int64_t w = idx % W, h = (idx / W) % H, t = (idx / (W * H)) % Tn, b = idx / (W * H * Tn);
+	T qv = q[idx], acc = 0;
+	for (int64_t s = 0; s < Tn; s++) {
+		T ws = sgn_exact(qv - k[((b * Tn + s) * H + h) * W + w]) * scale;
+		acc += ws * dA[((b * Tn + s) * Tn + t) * H + h];
+	}
+	dq[idx] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict__ dA, const T* __restrict__ q,
+                                                              const T* __restrict__ k, T* __restrict__ dk,
+                                                              int64_t B, int64_t Tn, int64_t H, int64_t W, T scale)
+{
+	int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= B * Tn * H * W) return;
+	int64_t w = idx % W, h = (idx / W) % H, s = (idx / (W * H)) % Tn, b = idx / (W * H * Tn);
+	T kv = k[idx], acc = 0;
+	for (int64_t t = 0; t < Tn; t++) {
+		T ws = sgn_exact(q[((b * Tn + t) * H + h) * W + w] - kv) * scale;
+		acc -= ws * dA[((b * Tn + s) * Tn + t) * H + h];
+	}
+	dk[idx] = acc;
+}
+
+// ------------------------------------------------------------------------------------------
+// fp32 forward, fast path
+// ------------------------------------------------------------------------------------------
+
+constexpr int FWD_SJ = 8;  // src rows finished between two output flushes
+
+// grid.x = dst tiles of 64 tokens, grid.y = src chunks, grid.z = B * head groups.
+// block = 64 * NW threads, NW = heads per group (<= 16); wave w of the block owns head hg*NW + w.
+// W is a compile-time multiple of 16; q and k must be 16-byte aligned.
+template <int W>
+__global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restrict__ q, const float* __restrict__ k,
+                                                             float* __restrict__ attn, int Tn, int H, int n_hg,
+                                                             int s_chunk, float scale)
+{
+	__shared__ float tile[FWD_SJ][WAVE * 17];
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int NW = blockDim.x >> 6;
+	const int b = blockIdx.z / n_hg, hg = blockIdx.z % n_hg;
+	const int h = min(hg * NW + wave, H - 1);  // surplus waves of the last group redo head H-1, never stored
+	const int t0 = blockIdx.x * WAVE;
+	const int t = min(t0 + lane, Tn - 1);
+
+	float qr[W];
+	{
+		const float4* qp = reinterpret_cast<const float4*>(q + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = qp[w4];
+			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
+		}
+	}
+
+	// output role of this thread in the flush: element e = threadIdx.x of the [64 x NW] row tile
+	const int o_tl = threadIdx.x / NW, o_hh = threadIdx.x % NW;
+	const bool o_ok = (t0 + o_tl < Tn) && (hg * NW + o_hh < H);
+	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (t0 + o_tl)) * H + hg * NW + o_hh;
+	const int64_t o_pitch = (int64_t)Tn * H;
+
+	const int s_begin = blockIdx.y * s_chunk;
+	const int s_end = min(Tn, s_begin + s_chunk);
+	for (int s0 = s_begin; s0 < s_end; s0 += FWD_SJ) {
+#pragma unroll
+		for (int j = 0; j < FWD_SJ; j++) {
+			const int s = min(s0 + j, Tn - 1);
+			const float* kp = k + (((int64_t)b * Tn + s) * H + h) * (int64_t)W;  // wave-uniform -> scalar loads
+			float a = 0.0f;
+#pragma unroll
+			for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
+			tile[j][lane * 17 + wave] = a * scale;
+		}
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < FWD_SJ; j++) {
+			const int s = s0 + j;
+			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * 17 + o_hh];
+		}
+		__syncthreads();
+	}
+}
+
+// ------------------------------------------------------------------------------------------
+// fp32 backward, fast path
+// ------------------------------------------------------------------------------------------
+
+constexpr int BWD_TT = 32;          // dst tokens per workgroup (register-resident q and dq)
+constexpr int BWD_SJ = 4;           // src tokens per staging step
+constexpr int BWD_TTP = BWD_TT + 4; // LDS row pitch: keeps 16-byte alignment for ds_read_b128
+constexpr float BWD_PRESCALE = 18446744073709551616.0f;  // 2^64
+
+// sign(x) for pre-scaled differences: x is (q-k)*2^64, so every non-zero difference of
+// magnitude >= 2^-64 saturates to +-1 and an exact tie stays 0.
+//
+// Four pair-elements of the backward pass (one src token against four dst tokens):
+//   sg = sign(qc_u - kc); dq_u += sg*g_u; dk -= sg*g_u.
+// One asm block so that the VALU instructions stay together: left to the compiler, the
+// accumulations are sunk away from the signs and the signs spill.
+__device__ __forceinline__ void pair_step4(const float* qc, float kc, const float4& g, float* dq, float& dk)
+{
+	float e0, e1;
+	asm volatile(
+	    "v_sub_f32 %0, %7, %11\n\t"
+	    "v_sub_f32 %1, %8, %11\n\t"
+	    "v_med3_f32 %0, %0, -1.0, 1.0\n\t"
+	    "v_med3_f32 %1, %1, -1.0, 1.0\n\t"
+	    "v_fmac_f32 %2, %0, %12\n\t"
+	    "v_fma_f32 %6, -%0, %12, %6\n\t"
+	    "v_fmac_f32 %3, %1, %13\n\t"
+	    "v_fma_f32 %6, -%1, %13, %6\n\t"
+	    "v_sub_f32 %0, %9, %11\n\t"
+	    "v_sub_f32 %1, %10, %11\n\t"
+	    "v_med3_f32 %0, %0, -1.0, 1.0\n\t"
+	    "v_med3_f32 %1, %1, -1.0, 1.0\n\t"
+	    "v_fmac_f32 %4, %0, %14\n\t"
+	    "v_fma_f32 %6, -%0, %14, %6\n\t"
+	    "v_fmac_f32 %5, %1, %15\n\t"
+	    "v_fma_f32 %6, -%1, %15, %6"
+	    : "=&v"(e0), "=&v"(e1), "+v"(dq[0]), "+v"(dq[1]), "+v"(dq[2]), "+v"(dq[3]), "+v"(dk)
+	    : "v"(qc[0]), "v"(qc[1]), "v"(qc[2]), "v"(qc[3]), "v"(kc), "v"(g.x), "v"(g.y), "v"(g.z), "v"(g.w));
+}
+
+// grid.x = dst tiles, grid.y = column chunks of blockDim.x, grid.z = batches of this launch.
+// dkp: [n_ttiles][nb][T][HW] partials (or dk itself when there is a single dst tile).
+__global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restrict__ dA, const float* __restrict__ q,
+                                                             const float* __restrict__ k, float* __restrict__ dq,
+                                                             float* __restrict__ dkp, int Tn, int H, int W, float scale)
+{
+	extern __shared__ float gl[];  // [BWD_SJ][H][BWD_TTP]
+	const unsigned HW = (unsigned)(H * W);
+	const unsigned col_raw = blockIdx.y * blockDim.x + threadIdx.x;
+	// lanes past the last column shadow column 0: same inputs, same arithmetic, and they store
+	// the same bits to the same addresses as the lane that owns column 0
+	const unsigned col = col_raw < HW ? col_raw : 0u;
+	const int h = (int)(col / (unsigned)W);
+	const int b = blockIdx.z, nb = gridDim.z;
+	const int tt = blockIdx.x, t0 = tt * BWD_TT;
+	// wave-uniform row bases; lanes add the 32-bit column
+	const float* const q_b = q + (int64_t)b * Tn * HW;
+	const float* const k_b = k + (int64_t)b * Tn * HW;
+	const float* const dA_b = dA + (int64_t)b * Tn * Tn * H;
+	float* const dkp_b = dkp + ((int64_t)tt * nb + b) * Tn * HW;
+
+	float qc[BWD_TT], dqa[BWD_TT];
+#pragma unroll
+	for (int i = 0; i < BWD_TT; i++) {
+		const int t = min(t0 + i, Tn - 1);
+		qc[i] = (q_b + (int64_t)t * HW)[col] * BWD_PRESCALE;
+		dqa[i] = 0.0f;
+	}
+
+	const int n_stage = BWD_SJ * BWD_TT * H;  // floats staged per step
+	for (int s0 = 0; s0 < Tn; s0 += BWD_SJ) {
+		__syncthreads();
+		// stage dA[b, s0+j, t0+i, h] -> gl[(j*H + h)*TTP + i]; global order is (j, i, h)
+		for (int e = threadIdx.x; e < n_stage; e += blockDim.x) {
+			const int j = e / (BWD_TT * H), r = e % (BWD_TT * H);
+			const int i = r / H, hh = r % H;
+			const int s = s0 + j, t = t0 + i;
+			float g = 0.0f;
+			if (s < Tn && t < Tn) g = (dA_b + ((int64_t)s * Tn + t0) * H)[r];
+			gl[(j * H + hh) * BWD_TTP + i] = g;
+		}
+		float kc[BWD_SJ], dka[BWD_SJ];
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) {
+			const int s = min(s0 + j, Tn - 1);
+			kc[j] = (k_b + (int64_t)s * HW)[col] * BWD_PRESCALE;
+			dka[j] = 0.0f;
+		}
+		__syncthreads();
+		{
+			// all dA values of this step for the lane's head, read one float4 ahead of their use
+			const float4* gp0 = reinterpret_cast<const float4*>(gl + h * BWD_TTP);
+			constexpr int NI4 = BWD_TT / 4;
+			float4 g_cur = gp0[0];
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) {
+#pragma unroll
+				for (int i4 = 0; i4 < NI4; i4++) {
+					float4 g_nxt = g_cur;
+					if (i4 + 1 < NI4) g_nxt = gp0[(j * H * BWD_TTP) / 4 + i4 + 1];
+					else if (j + 1 < BWD_SJ) g_nxt = gp0[((j + 1) * H * BWD_TTP) / 4];
+					__builtin_amdgcn_sched_barrier(0);
+					pair_step4(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
+					g_cur = g_nxt;
+				}
+			}
+		}
+		// unconditional in the lane dimension: a store guarded by a per-lane predicate would let the
+		// compiler sink the dk chain into the guarded block and split the four-instruction groups
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) {
+			const int s = s0 + j;
+			if (s < Tn) (dkp_b + (int64_t)s * HW)[col] = dka[j] * scale;
+		}
+	}
+	float* const dq_b = dq + (int64_t)b * Tn * HW;
+#pragma unroll
+	for (int i = 0; i < BWD_TT; i++) {
+		const int t = t0 + i;
+		if (t < Tn) (dq_b + (int64_t)t * HW)[col] = dqa[i] * scale;
+	}
+}
+
+// dk[i] = sum over dst tiles, in tile order, of the partials; n = nb*T*HW elements per tile.
+// VEC: n and both base pointers are multiples of 4 floats.
+template <bool VEC>
+__global__ __launch_bounds__(256) void dense_bwd_reduce_dk(const float* __restrict__ dkp, float* __restrict__ dk,
+                                                             int64_t n, int n_tt)
+{
+	if (VEC) {
+		const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+		if (i >= n) return;
+		float4 acc = *reinterpret_cast<const float4*>(dkp + i);
+		for (int tt = 1; tt < n_tt; tt++) {
+			const float4 p = *reinterpret_cast<const float4*>(dkp + (int64_t)tt * n + i);
+			acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
+		}
+		*reinterpret_cast<float4*>(dk + i) = acc;
+	} else {
+		const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+		if (i >= n) return;
+		float acc = dkp[i];
+		for (int tt = 1; tt < n_tt; tt++) acc += dkp[(int64_t)tt * n + i];
+		dk[i] = acc;
+	}
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+
+bool shape_ok(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	return B >= 0 && T >= 0 && H >= 0 && W >= 0;
+}
+
+template <typename T>
+int launch_fwd_generic(const T* q, const T* k, T* attn, int64_t B, int64_t Tn, int64_t H, int64_t W, hipStream_t st)
+{
+	const T scale = (T)(-1.0 / sqrt((double)W));
+	dim3 grid((unsigned)l1_cdiv(Tn * H, 256), (unsigned)std::min<int64_t>(B * Tn, 65535), 1);
+	hipLaunchKernelGGL(dense_fwd_generic<T>, grid, dim3(256), 0, st, q, k, attn, B, Tn, H, W, scale);
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+template <typename T>
+int launch_bwd_generic(const T* dA, const T* q, const T* k, T* dq, T* dk, int64_t B, int64_t Tn, int64_t H,
+                       int64_t W, hipStream_t st)
+{
+	const T scale = (T)(-1.0 / sqrt((double)W));
+	const int64_t n = B * Tn * H * W;
+	dim3 grid((unsigned)l1_cdiv(n, 256));
+	hipLaunchKernelGGL(dense_bwd_generic_dq<T>, grid, dim3(256), 0, st, dA, q, k, dq, B, Tn, H, W, scale);
+	L1_LAUNCH_CHECK();
+	hipLaunchKernelGGL(dense_bwd_generic_dk<T>, grid, dim3(256), 0, st, dA, q, k, dk, B, Tn, H, W, scale);
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+// fast forward: W a multiple of 16 up to 128, 16-byte aligned rows, at least half a wave of tokens
+bool fwd_fast_ok(const float* q, const float* k, int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	if (W < 16 || W > 128 || (W % 16) != 0 || T < 32) return false;
+	if ((((uintptr_t)q) | ((uintptr_t)k)) & 15) return false;
+	const int64_t NW = H < 16 ? H : 16;
+	const int64_t n_hg = l1_cdiv(H, NW);
+	return B * n_hg <= 65535 && T <= (1 << 30) && H <= 65535;
+}
+
+int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int64_t Tn, int64_t H, int64_t W,
+                    hipStream_t st)
+{
+	const int NW = (int)(H < 16 ? H : 16);
+	const int n_hg = (int)l1_cdiv(H, NW);
+	const int n_tt = (int)l1_cdiv(Tn, WAVE);
+	// split the src range so that the launch has a few thousand workgroups, in multiples of FWD_SJ
+	int64_t want_chunks = l1_cdiv(2048, (int64_t)n_tt * B * n_hg);
+	int64_t s_chunk = l1_cdiv(l1_cdiv(Tn, want_chunks), FWD_SJ) * FWD_SJ;
+	if (s_chunk < 64) s_chunk = 64;
+	int n_sc = (int)l1_cdiv(Tn, s_chunk);
+	if (n_sc > 65535) { s_chunk = l1_cdiv(l1_cdiv(Tn, 65535), FWD_SJ) * FWD_SJ; n_sc = (int)l1_cdiv(Tn, s_chunk); }
+	const float scale = (float)(-1.0 / sqrt((double)W));
+	dim3 grid(n_tt, n_sc, (unsigned)(B * n_hg)), block(64 * NW);
+#define L1_FWD_CASE(WV)                                                                                          \
+	case WV:                                                                                                     \
+		hipLaunchKernelGGL(dense_fwd_f32_fast<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg,          \
+		                   (int)s_chunk, scale);                                                                 \
+		break
+	switch (W) {
+		L1_FWD_CASE(16); L1_FWD_CASE(32); L1_FWD_CASE(48); L1_FWD_CASE(64);
+		L1_FWD_CASE(80); L1_FWD_CASE(96); L1_FWD_CASE(112); L1_FWD_CASE(128);
+	default: return L1ATTN_ERR_ARG;
+	}
+#undef L1_FWD_CASE
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+struct BwdPlan {
+	bool fast;
+	int threads, n_cc, n_tt;
+	size_t lds_bytes;
+	size_t per_batch_bytes;  // partial-dk scratch for one batch (0 when a single dst tile)
+};
+
+BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	BwdPlan p{};
+	const int64_t HW = H * W;
+	p.lds_bytes = (size_t)BWD_SJ * H * BWD_TTP * sizeof(float);
+	p.fast = B >= 1 && T >= 16 && HW >= 32 && p.lds_bytes <= 64 * 1024 && T <= (1 << 30) && B <= 65535 &&
+	         HW <= (int64_t)1024 * 65535;
+	if (!p.fast) return p;
+	p.threads = (int)std::min<int64_t>(1024, l1_cdiv(HW, 64) * 64);
+	p.n_cc = (int)l1_cdiv(HW, p.threads);
+	p.n_tt = (int)l1_cdiv(T, BWD_TT);
+	p.per_batch_bytes = p.n_tt > 1 ? (size_t)p.n_tt * T * HW * sizeof(float) : 0;
+	return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+int l1attn_dense_fwd_f32(const float* q, const float* k, float* attn, int64_t B, int64_t T, int64_t H, int64_t W,
+                         void* stream)
+{
+	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	if (B * T * T * H == 0) return L1ATTN_OK;
+	if (!q || !k || !attn) return L1ATTN_ERR_ARG;
+	hipStream_t st = (hipStream_t)stream;
+	if (W < 1) return L1ATTN_ERR_ARG;
+	if (fwd_fast_ok(q, k, B, T, H, W)) return launch_fwd_fast(q, k, attn, B, T, H, W, st);
+	return launch_fwd_generic<float>(q, k, attn, B, T, H, W, st);
+}
+
+int l1attn_dense_fwd_f64(const double* q, const double* k, double* attn, int64_t B, int64_t T, int64_t H, int64_t W,
+                         void* stream)
+{
+	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	if (B * T * T * H == 0) return L1ATTN_OK;
+	if (!q || !k || !attn) return L1ATTN_ERR_ARG;
+	hipStream_t st = (hipStream_t)stream;
+	if (W < 1) return L1ATTN_ERR_ARG;
+	return launch_fwd_generic<double>(q, k, attn, B, T, H, W, st);
+}
+
+size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	if (!shape_ok(B, T, H, W) || B * T * H * W == 0) return 0;
+	BwdPlan p = bwd_plan(B, T, H, W);
+	if (!p.fast || p.per_batch_bytes == 0) return 0;
+	// enough batches per launch to put >= 1024 workgroups in flight, never more than B
+	int64_t nb = l1_cdiv(1024, (int64_t)p.n_tt * p.n_cc);
+	if (nb > B) nb = B;
+	return p.per_batch_bytes * (size_t)nb;
+}
+
+int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
+                         int64_t T, int64_t H, int64_t W, void* workspace, size_t workspace_bytes, void* stream)
+{
+	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	const int64_t n = B * T * H * W;
+	if (n == 0) return L1ATTN_OK;
+	if (!d_attn || !q || !k || !dq || !dk) return L1ATTN_ERR_ARG;
+	hipStream_t st = (hipStream_t)stream;
+	BwdPlan p = bwd_plan(B, T, H, W);
+	if (!p.fast) return launch_bwd_generic<float>(d_attn, q, k, dq, dk, B, T, H, W, st);
+	const float scale = (float)(-1.0 / sqrt((double)W));
+	const int64_t HW = H * W;
+	if (p.per_batch_bytes == 0) {
+		dim3 grid(1, p.n_cc, (unsigned)B);
+		hipLaunchKernelGGL(dense_bwd_f32_fast, grid, dim3(p.threads), p.lds_bytes, st, d_attn, q, k, dq, dk, (int)T,
+		                   (int)H, (int)W, scale);
+		L1_LAUNCH_CHECK();
+		return L1ATTN_OK;
+	}
+	if (!workspace || workspace_bytes < p.per_batch_bytes) return L1ATTN_ERR_WORKSPACE;
+	int64_t nb_max = (int64_t)(workspace_bytes / p.per_batch_bytes);
+	if (nb_max > B) nb_max = B;
+	float* dkp = (float*)workspace;
+	for (int64_t b0 = 0; b0 < B; b0 += nb_max) {
+		const int64_t nb = std::min<int64_t>(nb_max, B - b0);
+		dim3 grid(p.n_tt, p.n_cc, (unsigned)nb);
+		hipLaunchKernelGGL(dense_bwd_f32_fast, grid, dim3(p.threads), p.lds_bytes, st, d_attn + b0 * T * T * H,
+		                   q + b0 * T * HW, k + b0 * T * HW, dq + b0 * T * HW, dkp, (int)T, (int)H, (int)W, scale);
+		L1_LAUNCH_CHECK();
+		const int64_t ne = nb * T * HW;
+		const bool vec = ((T * HW) % 4 == 0) && ((((uintptr_t)dkp) | ((uintptr_t)dk)) & 15) == 0;
+		if (vec)
+			hipLaunchKernelGGL(dense_bwd_reduce_dk<true>, dim3((unsigned)l1_cdiv(ne, 1024)), dim3(256), 0, st, dkp,
+			                   dk + b0 * T * HW, ne, p.n_tt);
+		else
+			hipLaunchKernelGGL(dense_bwd_reduce_dk<false>, dim3((unsigned)l1_cdiv(ne, 256)), dim3(256), 0, st, dkp,
+			                   dk + b0 * T * HW, ne, p.n_tt);
+		L1_LAUNCH_CHECK();
+	}
+	return L1ATTN_OK;
+}
+
+int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k, double* dq, double* dk, int64_t B,
+                         int64_t T, int64_t H, int64_t W, void* workspace, size_t workspace_bytes, void* stream)
+{
+	(void)workspace; (void)workspace_bytes;
+	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	if (B * T * H * W == 0) return L1ATTN_OK;
+	if (!d_attn || !q || !k || !dq || !dk) return L1ATTN_ERR_ARG;
+	return launch_bwd_generic<double>(d_attn, q, k, dq, dk, B, T, H, W, (hipStream_t)stream);
+}
+
+}  // extern "C"

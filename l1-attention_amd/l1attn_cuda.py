@@ -1,0 +1,41 @@
+"""Drop-in for the reference module of the same name (cuda/l1attn_cuda.py:7-32): dense L1
+attention logits with autograd, computed by the gfx950 HIP library.
+
+    m = l1attn_cuda.L1Attn()
+    a = m(q, k)              # q,k [batch, n_ctx, n_heads, width] -> a [batch, src, dst, heads]
+    a_sm = F.softmax(a, 1)   # softmax over the SRC dimension (dim 1)
+    vo = torch.einsum('bsdh,bshw->bdhw', a_sm, v)
+
+a[b,s,t,h] = -1/sqrt(width) * sum_w |q[b,t,h,w] - k[b,s,h,w]|.
+"""
+import torch
+from torch import nn
+from torch.autograd import Function
+
+import _l1attn_hip as _drv
+
+
+class L1AttnFn(Function):
+    @staticmethod
+    def forward(ctx, q, k):
+        q = q.contiguous()
+        k = k.contiguous()
+        attn = _drv.dense_forward(q, k)
+        ctx.save_for_backward(q, k)
+        return attn[0]
+
+    @staticmethod
+    def backward(ctx, d_attn):
+        q, k = ctx.saved_tensors[:2]
+        # the reference driver rejects a non-contiguous d_attn (cuda/l1attn_cuda_drv.cpp:71);
+        # autograd may hand one over (e.g. an expanded gradient), so it is packed here instead
+        d_q, d_k = _drv.dense_backward(d_attn.contiguous(), q, k)
+        return d_q, d_k
+
+
+class L1Attn(nn.Module):
+    def __init__(self):
+        super(L1Attn, self).__init__()
+
+    def forward(self, q, k):
+        return L1AttnFn.apply(q, k)
