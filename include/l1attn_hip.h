@@ -67,6 +67,120 @@ int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k,
                          int64_t B, int64_t T, int64_t H, int64_t W,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* -------------------------------------------------------------------------- edge lists */
+
+/*
+ * expandCoo on the GPU: for an edge list co[E, co_stride>=2] of [dst, src] rows (device memory,
+ * 32- or 64-bit signed integers: co_bits = 32 | 64) writes coo int32 [E,4] (device) with
+ *   coo[i] = [dst_i, src_i, #{j<i : dst_j == dst_i}, #{j<i : src_j == src_i}]
+ * and mxlen_host[0..1] = {dst_mxlen, src_mxlen} = 1 + the largest rank of each kind ({1,1} for
+ * E == 0).  Replaces the Python loop expandCoo (python/l1attn_sparse.py:382-427;
+ * cuda/l1attn_sparse_cuda.py:58-101; cuda/l1attn_sparse_bidi_cuda.py:59-104;
+ * cpp/l1attn_sparse_cpp.py:61-106).  Bit-exact (integer only).  Because two host integers are
+ * returned, this call synchronises `stream` before returning.  Indices must be in
+ * [0, 2^31-1]: L1ATTN_ERR_INDEX otherwise (the reference's printed "degenerate sparse head"
+ * warnings are host-side diagnostics and are produced by the Python wrapper, not here).
+ * workspace: device memory, >= l1attn_expand_coo_workspace_bytes(E), 256-byte aligned.
+ */
+size_t l1attn_expand_coo_workspace_bytes(int64_t E);
+int l1attn_expand_coo(const void* co, int co_bits, int64_t co_stride, int64_t E,
+                      int32_t* coo, int32_t* mxlen_host,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Plan = the dst-sorted and src-sorted views of an edge list, built once per list and reused by
+ * every forward/backward on it.  It stands in for what the reference recomputes on every call
+ * through coo[:,2] (the dst_cnt slot of each edge in the padded [B,T,dst_mxlen,H] tensor,
+ * cuda/l1attn_sparse_cuda_kernel.cu:50-84) and replaces the atomicAdd scatters (:179, :232,
+ * :367-368, :568-569, :625-626) with segment walks.  Only columns 0 and 1 of coo are read
+ * (coo int32 [E, coo_stride>=2], device); slot order inside a segment is the original row order,
+ * i.e. the order of the reference's dst_cnt / src_cnt.  Rows with an index outside [0,T) are
+ * dropped and flagged (the reference's behaviour is undefined there).
+ * plan: device buffer of l1attn_sparse_plan_bytes(E,T) bytes, 256-byte aligned, opaque.
+ * l1attn_sparse_plan_build is asynchronous; l1attn_sparse_plan_check copies the 16-word header to
+ * header_host, synchronises, and returns L1ATTN_ERR_INDEX if rows were dropped
+ * (header words: 1 = E, 2 = T, 3 = dropped flag, 4 = longest dst segment, 5 = longest src segment).
+ */
+size_t l1attn_sparse_plan_bytes(int64_t E, int64_t T);
+size_t l1attn_sparse_plan_workspace_bytes(int64_t E, int64_t T);
+int l1attn_sparse_plan_build(const int32_t* coo, int64_t coo_stride, int64_t E, int64_t T,
+                             void* plan, size_t plan_bytes,
+                             void* workspace, size_t workspace_bytes, void* stream);
+int l1attn_sparse_plan_check(const void* plan, int64_t E, int64_t T, int32_t* header_host, void* stream);
+
+/* ----------------------------------------------------------------------------- sparse */
+
+/*
+ * Sparse L1 attention over an edge list (plan from l1attn_sparse_plan_build for the same E, T):
+ *   a_c = -1/sqrt(W) * sum_w |q[b,dst_c,h,w] - k[b,src_c,h,w]|
+ *   p_c = exp(a_c) / (1 + sum_{c': dst_c' = dst_c} exp(a_c'))   if use_softmax, else exp(a_c)
+ *   vo[b,dst,h,:] = sum_{c: dst_c = dst} p_c * v[b,src_c,h,:]        (0 for a dst without edges)
+ * Replaces l1attn_sparse_cuda_drv.forward(v,q,k,coo,dst_mxlen,use_softmax) -> [vo, attn]
+ * (cuda/l1attn_sparse_cuda_drv.cpp:32-46, kernels cuda/l1attn_sparse_cuda_kernel.cu:27-181,
+ * launcher :373-445; CPU twin cpp/l1attn_sparse_drv.cpp:13-91).
+ * q,k [B,T,H,W]; v,vo [B,T,H,Wv].  P [B,E,H] receives the edge weights p_c in plan slot order; it
+ * is the saved-for-backward tensor that the reference returns as the padded `attn`
+ * [B,T,dst_mxlen,H].  dst_mxlen is not needed: segments carry their own length.
+ * Limits: max(W,Wv) <= 1024 when both are multiples of 4 and all pointers 16-byte aligned,
+ * else <= 256 (L1ATTN_ERR_RANGE beyond).
+ */
+int l1attn_sparse_fwd_f32(const float* v, const float* q, const float* k, const void* plan,
+                          float* vo, float* P,
+                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                          int use_softmax, void* stream);
+int l1attn_sparse_fwd_f64(const double* v, const double* q, const double* k, const void* plan,
+                          double* vo, double* P,
+                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                          int use_softmax, void* stream);
+
+/*
+ * Backward of the above: dv[b,src] = sum p_c*dvo[b,dst]; dp_c = v[b,src].dvo[b,dst];
+ * da_c = p_c*(dp_c - sum_c' p_c' dp_c') (softmax) or p_c*dp_c; dq[b,dst] += scale*sign(q-k)*da_c;
+ * dk[b,src] -= scale*sign(q-k)*da_c.  Replaces l1attn_sparse_cuda_drv.backward(dvo,v,q,k,coo,attn,
+ * dst_mxlen,use_softmax) -> [dv,dq,dk] (cuda/l1attn_sparse_cuda_drv.cpp:48-69, kernels
+ * cuda/l1attn_sparse_cuda_kernel.cu:183-370, launcher :447-531; CPU twin
+ * cpp/l1attn_sparse_drv.cpp:93-190; the O(dst_mxlen^2) Jacobian loop :152-167 is evaluated in closed
+ * form).  DA [B,E,H] is scratch for da_c (caller-owned, contents undefined on return).
+ * Deterministic: no atomics.
+ */
+int l1attn_sparse_bwd_f32(const float* dvo, const float* v, const float* q, const float* k,
+                          const void* plan, const float* P,
+                          float* dv, float* dq, float* dk, float* DA,
+                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                          int use_softmax, void* stream);
+int l1attn_sparse_bwd_f64(const double* dvo, const double* v, const double* q, const double* k,
+                          const void* plan, const double* P,
+                          double* dv, double* dq, double* dk, double* DA,
+                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                          int use_softmax, void* stream);
+
+/*
+ * Bidirectional variant: vo[b,dst] += p_c*vf[b,src] and vo[b,src] += p_c*vb[b,dst]; backward
+ * dvf[b,src] += p_c*dvo[b,dst], dvb[b,dst] += p_c*dvo[b,src],
+ * dp_c = vf[b,src].dvo[b,dst] + vb[b,dst].dvo[b,src]; dq, dk as above.
+ * Replaces l1attn_sparse_bidi_cuda_drv.forward / .backward
+ * (cuda/l1attn_sparse_bidi_cuda_drv.cpp:34-80, kernels cuda/l1attn_sparse_cuda_kernel.cu:535-649,
+ * launchers :651-815; CPU twin cpp/l1attn_sparse_bidi_drv.cpp:15-212).
+ */
+int l1attn_sparse_bidi_fwd_f32(const float* vf, const float* vb, const float* q, const float* k,
+                               const void* plan, float* vo, float* P,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                               int use_softmax, void* stream);
+int l1attn_sparse_bidi_fwd_f64(const double* vf, const double* vb, const double* q, const double* k,
+                               const void* plan, double* vo, double* P,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                               int use_softmax, void* stream);
+int l1attn_sparse_bidi_bwd_f32(const float* dvo, const float* vf, const float* vb, const float* q,
+                               const float* k, const void* plan, const float* P,
+                               float* dvf, float* dvb, float* dq, float* dk, float* DA,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                               int use_softmax, void* stream);
+int l1attn_sparse_bidi_bwd_f64(const double* dvo, const double* vf, const double* vb, const double* q,
+                               const double* k, const void* plan, const double* P,
+                               double* dvf, double* dvb, double* dq, double* dk, double* DA,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                               int use_softmax, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -45,6 +45,25 @@ def lib():
             f = getattr(L, "l1attn_dense_bwd_" + sfx)
             f.restype = ctypes.c_int
             f.argtypes = [_c_p] * 5 + [_c_i64] * 4 + [_c_p, _c_sz, _c_p]
+        _c_i = ctypes.c_int
+        L.l1attn_expand_coo_workspace_bytes.restype = _c_sz
+        L.l1attn_expand_coo_workspace_bytes.argtypes = [_c_i64]
+        L.l1attn_expand_coo.restype = _c_i
+        L.l1attn_expand_coo.argtypes = [_c_p, _c_i, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_sz, _c_p]
+        for n in ("l1attn_sparse_plan_bytes", "l1attn_sparse_plan_workspace_bytes"):
+            getattr(L, n).restype = _c_sz
+            getattr(L, n).argtypes = [_c_i64, _c_i64]
+        L.l1attn_sparse_plan_build.restype = _c_i
+        L.l1attn_sparse_plan_build.argtypes = [_c_p, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p, _c_sz, _c_p]
+        L.l1attn_sparse_plan_check.restype = _c_i
+        L.l1attn_sparse_plan_check.argtypes = [_c_p, _c_i64, _c_i64, _c_p, _c_p]
+        dims = [_c_i64] * 6 + [_c_i, _c_p]
+        for sfx in ("f32", "f64"):
+            for name, nptr in (("l1attn_sparse_fwd_", 6), ("l1attn_sparse_bwd_", 10),
+                               ("l1attn_sparse_bidi_fwd_", 7), ("l1attn_sparse_bidi_bwd_", 12)):
+                f = getattr(L, name + sfx)
+                f.restype = _c_i
+                f.argtypes = [_c_p] * nptr + dims
         _lib = L
     return _lib
 
@@ -118,3 +137,171 @@ def dense_backward(d_attn, q, k):
             ptr(ws) if ws is not None else None, ws_bytes, stream_of(q))
     check(rc, "l1attn_dense_bwd_" + sfx)
     return [dq, dk]
+
+
+# ------------------------------------------------------------------------------- edge lists
+
+def expand_coo(co):
+    """GPU expandCoo: co [E,2] integer [dst,src] rows -> (coo int32 [E,4] on co.device, dst_mxlen,
+    src_mxlen).  python/l1attn_sparse.py:382-427.  A CPU `co` is copied to the current GPU and the
+    result copied back, as the reference returns `coo` on co.device."""
+    if co.dim() != 2 or co.shape[1] < 2:
+        raise RuntimeError("co must be [cl, 2] rows of [dst, src]")
+    if co.dtype not in (torch.int8, torch.uint8, torch.int16, torch.int32, torch.int64):
+        raise RuntimeError("co must hold integers, got %s" % co.dtype)
+    dev = co.device if co.is_cuda else torch.device("cuda", torch.cuda.current_device())
+    cod = co.to(dev)
+    if cod.dtype not in (torch.int32, torch.int64):
+        cod = cod.to(torch.int64)
+    cod = cod.contiguous()
+    E = cod.shape[0]
+    coo = torch.zeros((E, 4), dtype=torch.int32, device=dev)
+    mx = (ctypes.c_int32 * 2)()
+    L = lib()
+    with torch.cuda.device(dev):
+        ws_bytes = L.l1attn_expand_coo_workspace_bytes(E)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        rc = L.l1attn_expand_coo(ptr(cod), 64 if cod.dtype == torch.int64 else 32, cod.shape[1], E,
+                                 ptr(coo), mx, ptr(ws), ws_bytes, stream_of(cod))
+    check(rc, "l1attn_expand_coo")
+    if not co.is_cuda:
+        coo = coo.cpu()
+    return coo, int(mx[0]), int(mx[1])
+
+
+class Plan(object):
+    """dst- and src-sorted views of one edge list on one device (opaque device buffer)."""
+    __slots__ = ("buf", "E", "T", "max_dst_deg", "max_src_deg")
+
+
+def build_plan(coo, n_tok):
+    """Plan for coo [E, >=2] int32 (device) over n_tok tokens.  Raises on an index outside [0, n_tok)."""
+    E = coo.shape[0]
+    L = lib()
+    plan = Plan()
+    with torch.cuda.device(coo.device):
+        nbytes = L.l1attn_sparse_plan_bytes(E, n_tok)
+        plan.buf = torch.empty(nbytes, dtype=torch.uint8, device=coo.device)
+        ws_bytes = L.l1attn_sparse_plan_workspace_bytes(E, n_tok)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=coo.device)
+        st = stream_of(coo)
+        rc = L.l1attn_sparse_plan_build(ptr(coo), coo.shape[1], E, n_tok, ptr(plan.buf), nbytes,
+                                        ptr(ws), ws_bytes, st)
+        check(rc, "l1attn_sparse_plan_build")
+        hdr = (ctypes.c_int32 * 16)()
+        rc = L.l1attn_sparse_plan_check(ptr(plan.buf), E, n_tok, hdr, st)
+    check(rc, "l1attn_sparse_plan_check")
+    plan.E, plan.T = E, n_tok
+    plan.max_dst_deg, plan.max_src_deg = int(hdr[4]), int(hdr[5])
+    return plan
+
+
+def plan_for(coo, n_tok):
+    """The plan of `coo`, cached on the tensor object and invalidated by in-place writes to it."""
+    check_input(coo, "coo")
+    if coo.dtype != torch.int32 or coo.dim() != 2 or coo.shape[1] < 2:
+        raise RuntimeError("coo must be an int32 [cl, >=2] tensor (the output of expandCoo)")
+    cached = getattr(coo, "_l1attn_plan", None)
+    key = (coo._version, coo.data_ptr(), tuple(coo.shape), int(n_tok))
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    plan = build_plan(coo, int(n_tok))
+    try:
+        coo._l1attn_plan = (key, plan)
+    except AttributeError:
+        pass
+    return plan
+
+
+# ----------------------------------------------------------------------------------- sparse
+
+def _sparse_shapes(v, q, k):
+    if q.dim() != 4 or q.shape != k.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
+        raise RuntimeError("v, q, k must be [batch, n_tok, n_heads, width] tensors with equal leading dims")
+    if not (v.dtype == q.dtype == k.dtype) or not (v.device == q.device == k.device):
+        raise RuntimeError("v, q, k must share dtype and device")
+    B, T, H, W = q.shape
+    return B, T, H, W, v.shape[3]
+
+
+def sparse_forward(v, q, k, coo, dst_mxlen, use_softmax, plan=None):
+    """l1attn_sparse_cuda_drv.forward(v,q,k,coo,dst_mxlen,use_softmax) -> [vo, attn]
+    (cuda/l1attn_sparse_cuda_drv.cpp:32-46).  The second tensor is the edge-weight tensor P [B,E,H]
+    in plan slot order (the reference's padded attn is internal to its backward).  dst_mxlen is
+    accepted for signature compatibility; segment lengths come from the plan."""
+    for x, n in ((v, "v"), (q, "q"), (k, "k"), (coo, "coo")):
+        check_input(x, n)
+    B, T, H, W, Wv = _sparse_shapes(v, q, k)
+    if plan is None:
+        plan = plan_for(coo, T)
+    E = plan.E
+    sfx = sfx_of(q)
+    vo = torch.empty_like(v)
+    P = torch.empty((B, E, H), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = getattr(lib(), "l1attn_sparse_fwd_" + sfx)(
+            ptr(v), ptr(q), ptr(k), ptr(plan.buf), ptr(vo), ptr(P), B, T, H, W, Wv, E,
+            int(bool(use_softmax)), stream_of(q))
+    check(rc, "l1attn_sparse_fwd_" + sfx)
+    return [vo, P]
+
+
+def sparse_backward(dvo, v, q, k, coo, P, dst_mxlen, use_softmax, plan=None):
+    """l1attn_sparse_cuda_drv.backward(dvo,v,q,k,coo,attn,dst_mxlen,use_softmax) -> [dv,dq,dk]
+    (cuda/l1attn_sparse_cuda_drv.cpp:48-69)."""
+    for x, n in ((dvo, "dvo"), (v, "v"), (q, "q"), (k, "k"), (coo, "coo"), (P, "attn")):
+        check_input(x, n)
+    B, T, H, W, Wv = _sparse_shapes(v, q, k)
+    if plan is None:
+        plan = plan_for(coo, T)
+    E = plan.E
+    sfx = sfx_of(q)
+    dv, dq, dk = torch.empty_like(v), torch.empty_like(q), torch.empty_like(k)
+    DA = torch.empty_like(P)
+    with torch.cuda.device(q.device):
+        rc = getattr(lib(), "l1attn_sparse_bwd_" + sfx)(
+            ptr(dvo), ptr(v), ptr(q), ptr(k), ptr(plan.buf), ptr(P), ptr(dv), ptr(dq), ptr(dk), ptr(DA),
+            B, T, H, W, Wv, E, int(bool(use_softmax)), stream_of(q))
+    check(rc, "l1attn_sparse_bwd_" + sfx)
+    return [dv, dq, dk]
+
+
+def bidi_forward(vf, vb, q, k, coo, dst_mxlen, use_softmax, plan=None):
+    """l1attn_sparse_bidi_cuda_drv.forward -> [vo, attn] (cuda/l1attn_sparse_bidi_cuda_drv.cpp:34-50)."""
+    for x, n in ((vf, "vf"), (vb, "vb"), (q, "q"), (k, "k"), (coo, "coo")):
+        check_input(x, n)
+    B, T, H, W, Wv = _sparse_shapes(vf, q, k)
+    if vb.shape != vf.shape or vb.dtype != vf.dtype:
+        raise RuntimeError("vf and vb must have one shape and dtype")
+    if plan is None:
+        plan = plan_for(coo, T)
+    E = plan.E
+    sfx = sfx_of(q)
+    vo = torch.empty_like(vf)
+    P = torch.empty((B, E, H), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = getattr(lib(), "l1attn_sparse_bidi_fwd_" + sfx)(
+            ptr(vf), ptr(vb), ptr(q), ptr(k), ptr(plan.buf), ptr(vo), ptr(P), B, T, H, W, Wv, E,
+            int(bool(use_softmax)), stream_of(q))
+    check(rc, "l1attn_sparse_bidi_fwd_" + sfx)
+    return [vo, P]
+
+
+def bidi_backward(dvo, vf, vb, q, k, coo, P, dst_mxlen, use_softmax, plan=None):
+    """l1attn_sparse_bidi_cuda_drv.backward -> [dvf,dvb,dq,dk] (cuda/l1attn_sparse_bidi_cuda_drv.cpp:52-75)."""
+    for x, n in ((dvo, "dvo"), (vf, "vf"), (vb, "vb"), (q, "q"), (k, "k"), (coo, "coo"), (P, "attn")):
+        check_input(x, n)
+    B, T, H, W, Wv = _sparse_shapes(vf, q, k)
+    if plan is None:
+        plan = plan_for(coo, T)
+    E = plan.E
+    sfx = sfx_of(q)
+    dvf, dvb, dq, dk = torch.empty_like(vf), torch.empty_like(vb), torch.empty_like(q), torch.empty_like(k)
+    DA = torch.empty_like(P)
+    with torch.cuda.device(q.device):
+        rc = getattr(lib(), "l1attn_sparse_bidi_bwd_" + sfx)(
+            ptr(dvo), ptr(vf), ptr(vb), ptr(q), ptr(k), ptr(plan.buf), ptr(P),
+            ptr(dvf), ptr(dvb), ptr(dq), ptr(dk), ptr(DA),
+            B, T, H, W, Wv, E, int(bool(use_softmax)), stream_of(q))
+    check(rc, "l1attn_sparse_bidi_bwd_" + sfx)
+    return [dvf, dvb, dq, dk]
