@@ -378,7 +378,8 @@ int l1attn_sparse_plan_build(const int32_t* coo, int64_t coo_stride, int64_t E, 
 		if (!workspace || workspace_bytes < 256) return L1ATTN_ERR_WORKSPACE;
 		stats = (int*)workspace;
 		hipLaunchKernelGGL(fill_words, dim3(1), dim3(64), 0, st, stats, ST_WORDS, 0);
-		const int n = (int)(2 * (T + 2));
+		// dst_ptr and src_ptr are adjacent arrays; zero both up to the start of csr_src
+		const int n = (int)(L.csr_src - L.dst_ptr);
 		hipLaunchKernelGGL(fill_words, dim3((unsigned)l1_cdiv(n, 256)), dim3(256), 0, st, words + L.dst_ptr, n, 0);
 		L1_LAUNCH_CHECK();
 		hipLaunchKernelGGL(plan_header, dim3(1), dim3(64), 0, st, words, 0, (int)T, stats, words + L.dst_ptr);
