@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the L1-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-sparse] [--skip-cpu]
+
+A step is one dense L1Attn forward + backward (through the reference's Python API,
+l1attn_cuda.L1AttnFn) over the headline configuration  q,k fp32 [B=8, T=4096, H=16, W=64],
+upstream gradient dA fp32 [8,4096,4096,16] ~ N(0,1), all resident in HBM before the timed region.
+Prints ONE JSON line: dense fwd+bwd throughput in GOP/s (algorithmic operations: 2 per
+pair-element forward, 4 backward, N = B*T*T*H*W pair-elements), the roofline of the dominant
+launch (the backward), the sparse / bidirectional-sparse / expandCoo figures of configurations 4
+and 5, and a CPU baseline timed on this box's host cores on a bounded sample of the same workload.
+Progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "l1-attention_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+P_VALU_TOPS = 78.6     # 256 CU x 4 SIMD x 16 lanes x 2 (packed fp32) x 2.4 GHz; the 157.3 TFLOP/s figure counts FMA as 2
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+# HBM bytes per dense-backward launch (B=8,T=4096,H=16,W=64) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# scaled by a copy kernel of known size; None until measured (see profiles/).
+DENSE_BWD_TRAFFIC_BYTES = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def dense_headline(steps, warmup):
+    import torch
+    import l1attn_cuda
+    B, T, H, W = 8, 4096, 16, 64
+    dev = torch.device("cuda:0")
+    import workloads
+    q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
+    q, k = q.to(dev).requires_grad_(), k.to(dev).requires_grad_()
+    gen = torch.Generator(device=dev).manual_seed(1002)
+    dA = torch.empty(B, T, T, H, device=dev)
+    for b in range(B):  # 8 GiB, generated on the device one batch at a time
+        dA[b].normal_(generator=gen)
+    N = B * T * T * H * W
+
+    def step(ev=None):
+        q.grad = None
+        k.grad = None
+        if ev:
+            ev[0].record()
+        a = l1attn_cuda.L1AttnFn.apply(q, k)
+        if ev:
+            ev[1].record()
+        a.backward(dA)
+        if ev:
+            ev[2].record()
+        del a
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    ms_per_step = wall * 1e3 / steps
+    out = {
+        "B": B, "T": T, "H": H, "W": W, "pair_elements": N,
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "ms_per_step": ms_per_step,
+        "fwd_tops": 2 * N / fwd_ms / 1e9, "bwd_tops": 4 * N / bwd_ms / 1e9,
+        "fwd_bwd_gops": 6 * N / (ms_per_step * 1e-3) / 1e9,
+    }
+    out["frac_of_valu_peak"] = out["fwd_bwd_gops"] / 1e3 / P_VALU_TOPS
+    del dA, q, k
+    torch.cuda.empty_cache()
+    return out
+
+
+def time_gpu(fn, iters, warm=2):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def sparse_configs(skip_cpu):
+    """Configuration 4 (one-directional, B4 T4096 H8 W32, degree U{1..64}) and configuration 5
+    (bidirectional, B1 T65536 H4 W64, Zipf degrees + self loops): fwd+bwd through the Python API."""
+    import torch
+    import workloads
+    import l1attn_sparse_cuda as sp
+    import l1attn_sparse_bidi_cuda as bi
+    from oracle import oracle
+    dev = torch.device("cuda:0")
+    res = {}
+    for name, bidi, (B, T, H, W), co in (
+            ("config4_uni", False, (4, 4096, 8, 32), workloads.uniform_degree_graph(4096, 64, seed=1004)),
+            ("config5_bidi", True, (1, 65536, 4, 64), workloads.powerlaw_graph(65536, seed=1005))):
+        E = co.shape[0]
+        cod = co.to(dev)
+        ms_expand = time_gpu(lambda: sp.expandCoo(cod, warn=False), 3, warm=1)
+        coo, dmx, smx = sp.expandCoo(cod, warn=False)
+        cpu_expand_ms = None
+        if not skip_cpu:
+            t0 = time.perf_counter()
+            ocoo, odmx, osmx = oracle.expand_coo(co)
+            cpu_expand_ms = (time.perf_counter() - t0) * 1e3
+            assert torch.equal(coo.cpu(), ocoo) and (dmx, smx) == (odmx, osmx)
+        x = [t.to(dev).requires_grad_() for t in workloads.sparse_inputs(B, T, H, W, seed=1004 + bidi, n=4)]
+        dvo = torch.randn(B, T, H, W, device=dev)
+        if bidi:
+            m = bi.L1AttnSparseBidi()
+            args = (x[0], x[1], x[2], x[3])
+        else:
+            m = sp.L1AttnSparse()
+            args = (x[0], x[2], x[3])
+
+        def fwd():
+            return m(*args, coo, dmx)
+
+        def fwdbwd():
+            for t in x:
+                t.grad = None
+            fwd().backward(dvo)
+
+        ms_fwd = time_gpu(fwd, 10)
+        ms = time_gpu(fwdbwd, 10)
+        r, g = B * H * W * 4, B * H * 4
+        if bidi:
+            bytes_alg = E * (8 * r + 7 * g + 64) + T * 11 * r
+        else:
+            bytes_alg = E * (6 * r + 5 * g + 48) + T * 8 * r
+        bytes_min = 11 * T * r + 16 * E + 2 * g * E
+        res[name] = {
+            "B": B, "T": T, "H": H, "W": W, "edges": E, "dst_mxlen": dmx, "src_mxlen": smx,
+            "fwd_ms": ms_fwd, "fwd_bwd_ms": ms,
+            "edges_per_s": E / (ms * 1e-3), "edge_heads_per_s": E * B * H / (ms * 1e-3),
+            "bytes_alg": bytes_alg, "alg_GBps": bytes_alg / (ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": bytes_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "bytes_min": bytes_min, "min_GBps": bytes_min / (ms * 1e-3) / 1e9,
+            "expand_coo_gpu_ms": ms_expand, "expand_coo_cpu_oracle_ms": cpu_expand_ms,
+            "note": "plan build (two radix sorts) is cached per edge list and excluded from fwd/bwd time",
+        }
+        log(name, json.dumps(res[name]))
+    return res
+
+
+def cpu_baseline():
+    """The reference's own CPU extension (oracle/_ref, fp64, one thread, scalar) when it was built and
+    carried here, else the C restatement (oracle/liboracle.so, fp64, one thread), on a bounded sample
+    of the headline workload: same H, W and input distribution, B=1 and T=1024 (1/128 of the pair-elements)."""
+    import torch
+    import workloads
+    from oracle import oracle
+    B, T, H, W = 1, 1024, 16, 64
+    q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
+    q, k = q.double(), k.double()
+    dA = torch.randn(B, T, T, H, generator=torch.Generator().manual_seed(1002), dtype=torch.float64)
+    N = B * T * T * H * W
+    mods = None
+    try:
+        mods = oracle.ref_modules()
+    except Exception as e:  # an _ref built against another torch would fail to import
+        log("oracle/_ref not usable:", repr(e))
+    torch.set_num_threads(1)
+    oracle.set_threads(1)
+    if mods is not None:
+        kind = "reference"
+        t0 = time.perf_counter()
+        mods["l1attn_drv_cpp"].forward(q, k)
+        mods["l1attn_drv_cpp"].backward(dA, q, k)
+        dt = time.perf_counter() - t0
+    else:
+        kind = "port"
+        t0 = time.perf_counter()
+        oracle.dense_fwd(q, k)
+        oracle.dense_bwd(dA, q, k)
+        dt = time.perf_counter() - t0
+    # the same sample on all host cores with the OpenMP build of the restatement (fp32)
+    ncores = min(os.cpu_count() or 1, 16)
+    oracle.set_threads(ncores)
+    q32, k32, dA32 = q.float(), k.float(), dA.float()
+    t0 = time.perf_counter()
+    oracle.dense_fwd(q32, k32)
+    oracle.dense_bwd(dA32, q32, k32)
+    dt_mt = time.perf_counter() - t0
+    oracle.set_threads(1)
+    return {
+        "value": 6 * N / dt / 1e9, "unit": "GOP/s", "cores": 1, "kind": kind,
+        "sample": "dense fwd+bwd fp64, B=1 T=1024 H=16 W=64 (1/128 of the headline pair-elements), %.1f s" % dt,
+        "port_fp32_openmp": {"value": 6 * N / dt_mt / 1e9, "unit": "GOP/s", "cores": ncores,
+                             "note": "OpenMP over (batch, head) of the C restatement"},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--skip-sparse", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the hot path does not communicate; "
+              "see DESIGN.md for how it would shard); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    import _l1attn_hip
+    _l1attn_hip.lib()  # fail here, loudly, if the HIP library is not built
+
+    log("dense headline ...")
+    d = dense_headline(args.steps, args.warmup)
+    log(json.dumps(d))
+    N = d["pair_elements"]
+    roof = {
+        "bound": "valu", "kernel": "dense_bwd_f32_fast (+ dense_bwd_reduce_dk, one backward launch)",
+        "achieved": d["bwd_tops"], "peak": P_VALU_TOPS, "unit": "TFLOP/s",
+        "frac": d["bwd_tops"] / P_VALU_TOPS,
+        "traffic": DENSE_BWD_TRAFFIC_BYTES,
+        "flops_per_launch": 4 * N, "avg_launch_ms": d["bwd_ms"],
+        "note": "algorithmic ops (4 per pair-element) over the HIP-event time of the backward launch; "
+                "peak = packed-fp32 VALU issue rate, which this library does not use "
+                "(scalar-per-lane fp32 peaks at 39.3)",
+    }
+    out = {
+        "metric": "dense fwd+bwd GOP/s & % fp32 VALU peak; sparse fwd+bwd edges/s & HBM GB/s",
+        "value": d["fwd_bwd_gops"], "unit": "GOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": d["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "dense L1Attn fwd+bwd, q,k fp32 [B=8,T=4096,H=16,W=64], dA [8,4096,4096,16] "
+                               "(BASELINE.json configs[2], the headline dense configuration)",
+                   "B": 8, "T": 4096, "H": 16, "W": 64},
+        "frac_of_fp32_valu_peak": d["frac_of_valu_peak"],
+        "dense": d,
+        "roofline": roof,
+    }
+    if not args.skip_sparse:
+        log("sparse configurations ...")
+        out["sparse"] = sparse_configs(args.skip_cpu)
+    if not args.skip_cpu:
+        log("cpu baseline ...")
+        out["cpu_baseline"] = cpu_baseline()
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

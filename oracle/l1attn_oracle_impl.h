@@ -41,19 +41,20 @@ void FN(oracle_dense_fwd)(const REAL *q, const REAL *k, REAL *attn,
 }
 
 /* cpp/l1attn_drv.cpp:57-98.  d_attn [B,S,T,H]; dq,dk [B,T,H,W] (zero-initialised here).
- * Threads split over b only, so that every output element is accumulated by one
- * thread in the reference's own s,t order. */
+ * The reference nests b,s,t,h,w.  Here h is hoisted next to b so that OpenMP threads can split
+ * over (b,h): outputs of different heads are disjoint, and every output element is still
+ * accumulated by one thread in the reference's own (s,t) order, so the sums are unchanged. */
 void FN(oracle_dense_bwd)(const REAL *d_attn, const REAL *q, const REAL *k,
                           REAL *dq, REAL *dk, long B, long T, long H, long W)
 {
 	const REAL scale = (REAL)(-1.0 / sqrt((double)W));
 	memset(dq, 0, sizeof(REAL) * (size_t)(B * T * H * W));
 	memset(dk, 0, sizeof(REAL) * (size_t)(B * T * H * W));
-	#pragma omp parallel for schedule(static)
+	#pragma omp parallel for collapse(2) schedule(static)
 	for (long b = 0; b < B; b++) {
-		for (long s = 0; s < T; s++) {
-			for (long t = 0; t < T; t++) {
-				for (long h = 0; h < H; h++) {
+		for (long h = 0; h < H; h++) {
+			for (long s = 0; s < T; s++) {
+				for (long t = 0; t < T; t++) {
 					REAL d_a = d_attn[((b * T + s) * T + t) * H + h];
 					const REAL *qp = q + ((b * T + t) * H + h) * W;
 					const REAL *kp = k + ((b * T + s) * H + h) * W;
