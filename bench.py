@@ -217,6 +217,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--skip-sparse", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-dense", action="store_true", help="profiling aid: sparse legs only")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="profiling aid: only run three 1 GiB device-to-device copies, the known-size "
+                         "kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path does not communicate; "
@@ -228,6 +232,18 @@ def main():
         sys.exit(3)
     import _l1attn_hip
     _l1attn_hip.lib()  # fail here, loudly, if the HIP library is not built
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "copies": 3}))
+        return
+    if args.skip_dense:
+        print(json.dumps({"sparse": sparse_configs(True)}), flush=True)
+        return
 
     log("dense headline ...")
     d = dense_headline(args.steps, args.warmup)
