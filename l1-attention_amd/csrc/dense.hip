@@ -149,6 +149,108 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 	}
 }
 
+// Software-pipelined variant for W a multiple of 32.  The compiler schedules each scalar load of a
+// k chunk only a few instructions ahead of its first use, so every 16 floats a wave sits out a
+// scalar-cache/L2 round trip.  Here the k row streams through two 32-float SGPR buffers: the load of
+// chunk c+1 is issued before the 64 VALU instructions of chunk c, so one chunk of compute (times the
+// waves interleaved on the SIMD) covers the latency.  Scalar loads return out of order, hence the
+// only wait used is lgkmcnt(0).
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ void sload32(f32x16& lo, f32x16& hi, const float* p)
+{
+	// early-clobber outputs: the second load must still see the pointer
+	asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40" : "=&s"(lo), "=&s"(hi) : "s"(p));
+}
+__device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
+{
+	asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(lo), "+s"(hi));
+}
+
+template <int W>
+__global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restrict__ q, const float* __restrict__ k,
+                                                             float* __restrict__ attn, int Tn, int H, int n_hg,
+                                                             int s_chunk, float scale)
+{
+	static_assert(W % 32 == 0 && (FWD_SJ % 2) == 0, "chunk stream must keep buffer parity across src blocks");
+	__shared__ float tile[FWD_SJ][WAVE * 17];
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int NW = blockDim.x >> 6;
+	const int b = blockIdx.z / n_hg, hg = blockIdx.z % n_hg;
+	const int h = min(hg * NW + wave, H - 1);
+	const int t0 = blockIdx.x * WAVE;
+	const int t = min(t0 + lane, Tn - 1);
+
+	float qr[W];
+	{
+		const float4* qp = reinterpret_cast<const float4*>(q + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = qp[w4];
+			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
+		}
+	}
+	const int o_tl = threadIdx.x / NW, o_hh = threadIdx.x % NW;
+	const bool o_ok = (t0 + o_tl < Tn) && (hg * NW + o_hh < H);
+	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (t0 + o_tl)) * H + hg * NW + o_hh;
+	const int64_t o_pitch = (int64_t)Tn * H;
+
+	constexpr int CPR = W / 32;          // chunks per k row
+	constexpr int NCH = FWD_SJ * CPR;    // chunks per src block
+	const int64_t krow = (int64_t)H * W;  // floats between consecutive src rows
+	const float* const kb = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;  // row 0 of this (b,h), wave-uniform
+	// last chunk of the last row: the running prefetch pointer is clamped to it, so rows past the end
+	// of the tensor (computed but never stored) read valid memory
+	const float* const k_last = kb + (int64_t)(Tn - 1) * krow + (CPR - 1) * 32;
+
+	const int s_begin = blockIdx.y * s_chunk;
+	const int s_end = min(Tn, s_begin + s_chunk);
+	f32x16 b0l, b0h, b1l, b1h;
+	const float* kp = kb + (int64_t)s_begin * krow;  // chunk being prefetched
+	sload32(b0l, b0h, kp);
+	__builtin_amdgcn_sched_barrier(0);
+	for (int s0 = s_begin; s0 < s_end; s0 += FWD_SJ) {
+		float a = 0.0f;
+#pragma unroll
+		for (int c = 0; c < NCH; c++) {
+			const int j = c / CPR, part = c % CPR;
+			kp += (part == CPR - 1) ? krow - (CPR - 1) * 32 : 32;
+			kp = kp < k_last ? kp : k_last;
+			if ((c & 1) == 0) {
+				swait32(b0l, b0h);
+				__builtin_amdgcn_sched_barrier(0);
+				sload32(b1l, b1h, kp);
+				__builtin_amdgcn_sched_barrier(0);
+				if (part == 0) a = 0.0f;
+#pragma unroll
+				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + i] - b0l[i]);
+#pragma unroll
+				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b0h[i]);
+			} else {
+				swait32(b1l, b1h);
+				__builtin_amdgcn_sched_barrier(0);
+				sload32(b0l, b0h, kp);
+				__builtin_amdgcn_sched_barrier(0);
+				if (part == 0) a = 0.0f;
+#pragma unroll
+				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + i] - b1l[i]);
+#pragma unroll
+				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b1h[i]);
+			}
+			if (part == CPR - 1) tile[j][lane * 17 + wave] = a * scale;
+		}
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < FWD_SJ; j++) {
+			const int s = s0 + j;
+			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * 17 + o_hh];
+		}
+		__syncthreads();
+	}
+	swait32(b0l, b0h);  // drain the last prefetch before the wave ends
+}
+
 // ------------------------------------------------------------------------------------------
 // fp32 backward, fast path
 // ------------------------------------------------------------------------------------------
@@ -353,14 +455,16 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 	if (n_sc > 65535) { s_chunk = l1_cdiv(l1_cdiv(Tn, 65535), FWD_SJ) * FWD_SJ; n_sc = (int)l1_cdiv(Tn, s_chunk); }
 	const float scale = (float)(-1.0 / sqrt((double)W));
 	dim3 grid(n_tt, n_sc, (unsigned)(B * n_hg)), block(64 * NW);
-#define L1_FWD_CASE(WV)                                                                                          \
+#define L1_FWD_CASE(KERNEL, WV)                                                                                  \
 	case WV:                                                                                                     \
-		hipLaunchKernelGGL(dense_fwd_f32_fast<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg,          \
-		                   (int)s_chunk, scale);                                                                 \
+		hipLaunchKernelGGL(KERNEL<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, (int)s_chunk,        \
+		                   scale);                                                                               \
 		break
 	switch (W) {
-		L1_FWD_CASE(16); L1_FWD_CASE(32); L1_FWD_CASE(48); L1_FWD_CASE(64);
-		L1_FWD_CASE(80); L1_FWD_CASE(96); L1_FWD_CASE(112); L1_FWD_CASE(128);
+		L1_FWD_CASE(dense_fwd_f32_fast, 16); L1_FWD_CASE(dense_fwd_f32_pipe, 32);
+		L1_FWD_CASE(dense_fwd_f32_fast, 48); L1_FWD_CASE(dense_fwd_f32_pipe, 64);
+		L1_FWD_CASE(dense_fwd_f32_fast, 80); L1_FWD_CASE(dense_fwd_f32_fast, 96);
+		L1_FWD_CASE(dense_fwd_f32_fast, 112); L1_FWD_CASE(dense_fwd_f32_fast, 128);
 	default: return L1ATTN_ERR_ARG;
 	}
 #undef L1_FWD_CASE
