@@ -293,6 +293,10 @@ __device__ __forceinline__ void pair_step4(const float* qc, float kc, const floa
 
 // grid.x = dst tiles, grid.y = column chunks of blockDim.x, grid.z = batches of this launch.
 // dkp: [n_ttiles][nb][T][HW] partials (or dk itself when there is a single dst tile).
+// PER = staged dA values per thread and step (ceil(BWD_SJ*BWD_TT*H / blockDim.x) <= PER).  The dA and
+// k values of step n+1 are fetched into registers before the math of step n, so their latency is
+// covered by a whole step of VALU work.
+template <int PER>
 __global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restrict__ dA, const float* __restrict__ q,
                                                              const float* __restrict__ k, float* __restrict__ dq,
                                                              float* __restrict__ dkp, int Tn, int H, int W, float scale)
@@ -309,7 +313,7 @@ __global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restri
 	// wave-uniform row bases; lanes add the 32-bit column
 	const float* const q_b = q + (int64_t)b * Tn * HW;
 	const float* const k_b = k + (int64_t)b * Tn * HW;
-	const float* const dA_b = dA + (int64_t)b * Tn * Tn * H;
+	const float* const dA_b = dA + ((int64_t)b * Tn * Tn + t0) * H;
 	float* const dkp_b = dkp + ((int64_t)tt * nb + b) * Tn * HW;
 
 	float qc[BWD_TT], dqa[BWD_TT];
@@ -320,26 +324,46 @@ __global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restri
 		dqa[i] = 0.0f;
 	}
 
-	const int n_stage = BWD_SJ * BWD_TT * H;  // floats staged per step
-	for (int s0 = 0; s0 < Tn; s0 += BWD_SJ) {
-		__syncthreads();
-		// stage dA[b, s0+j, t0+i, h] -> gl[(j*H + h)*TTP + i]; global order is (j, i, h)
-		for (int e = threadIdx.x; e < n_stage; e += blockDim.x) {
-			const int j = e / (BWD_TT * H), r = e % (BWD_TT * H);
-			const int i = r / H, hh = r % H;
-			const int s = s0 + j, t = t0 + i;
-			float g = 0.0f;
-			if (s < Tn && t < Tn) g = (dA_b + ((int64_t)s * Tn + t0) * H)[r];
-			gl[(j * H + hh) * BWD_TTP + i] = g;
+	// staging roles of this thread: element e = threadIdx.x + r*blockDim.x of the [j][i][hh] step tile
+	const int n_stage = BWD_SJ * BWD_TT * H;
+	int st_j[PER], st_lds[PER];
+	int64_t st_off[PER];
+	bool st_ok[PER];
+#pragma unroll
+	for (int r = 0; r < PER; r++) {
+		const int e = threadIdx.x + r * blockDim.x;
+		const int j = e / (BWD_TT * H), rr = e % (BWD_TT * H);
+		const int i = rr / H, hh = rr % H;
+		st_j[r] = j;
+		st_ok[r] = e < n_stage && t0 + i < Tn;
+		st_off[r] = (int64_t)j * Tn * H + rr;
+		st_lds[r] = e < n_stage ? (j * H + hh) * BWD_TTP + i : -1;
+	}
+	float g_pre[PER], k_pre[BWD_SJ];
+	auto prefetch = [&](int s0) {
+#pragma unroll
+		for (int r = 0; r < PER; r++) {
+			g_pre[r] = 0.0f;
+			if (st_ok[r] && s0 + st_j[r] < Tn) g_pre[r] = (dA_b + (int64_t)s0 * Tn * H)[st_off[r]];
 		}
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) k_pre[j] = (k_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
+	};
+	prefetch(0);
+
+	for (int s0 = 0; s0 < Tn; s0 += BWD_SJ) {
+		__syncthreads();  // the previous step's LDS reads are done
+#pragma unroll
+		for (int r = 0; r < PER; r++)
+			if (st_lds[r] >= 0) gl[st_lds[r]] = g_pre[r];
 		float kc[BWD_SJ], dka[BWD_SJ];
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) {
-			const int s = min(s0 + j, Tn - 1);
-			kc[j] = (k_b + (int64_t)s * HW)[col] * BWD_PRESCALE;
+			kc[j] = k_pre[j] * BWD_PRESCALE;
 			dka[j] = 0.0f;
 		}
 		__syncthreads();
+		if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
 		{
 			// all dA values of this step for the lane's head, read one float4 ahead of their use
 			const float4* gp0 = reinterpret_cast<const float4*>(gl + h * BWD_TTP);
@@ -474,7 +498,7 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 
 struct BwdPlan {
 	bool fast;
-	int threads, n_cc, n_tt;
+	int threads, n_cc, n_tt, per;
 	size_t lds_bytes;
 	size_t per_batch_bytes;  // partial-dk scratch for one batch (0 when a single dst tile)
 };
@@ -490,8 +514,24 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.threads = (int)std::min<int64_t>(1024, l1_cdiv(HW, 64) * 64);
 	p.n_cc = (int)l1_cdiv(HW, p.threads);
 	p.n_tt = (int)l1_cdiv(T, BWD_TT);
+	p.per = (int)l1_cdiv((int64_t)BWD_SJ * BWD_TT * H, p.threads);
+	if (p.per > 16) { p.fast = false; return p; }
 	p.per_batch_bytes = p.n_tt > 1 ? (size_t)p.n_tt * T * HW * sizeof(float) : 0;
 	return p;
+}
+
+void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* dA, const float* q, const float* k,
+                     float* dq, float* dkp, int T, int H, int W, float scale)
+{
+#define L1_BWD_CASE(PERV)                                                                                       \
+	hipLaunchKernelGGL(dense_bwd_f32_fast<PERV>, grid, dim3(p.threads), p.lds_bytes, st, dA, q, k, dq, dkp, T, H, W, \
+	                   scale)
+	if (p.per <= 1) L1_BWD_CASE(1);
+	else if (p.per <= 2) L1_BWD_CASE(2);
+	else if (p.per <= 4) L1_BWD_CASE(4);
+	else if (p.per <= 8) L1_BWD_CASE(8);
+	else L1_BWD_CASE(16);
+#undef L1_BWD_CASE
 }
 
 }  // namespace
@@ -546,8 +586,7 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 	const int64_t HW = H * W;
 	if (p.per_batch_bytes == 0) {
 		dim3 grid(1, p.n_cc, (unsigned)B);
-		hipLaunchKernelGGL(dense_bwd_f32_fast, grid, dim3(p.threads), p.lds_bytes, st, d_attn, q, k, dq, dk, (int)T,
-		                   (int)H, (int)W, scale);
+		launch_bwd_fast(p, grid, st, d_attn, q, k, dq, dk, (int)T, (int)H, (int)W, scale);
 		L1_LAUNCH_CHECK();
 		return L1ATTN_OK;
 	}
@@ -558,8 +597,8 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 	for (int64_t b0 = 0; b0 < B; b0 += nb_max) {
 		const int64_t nb = std::min<int64_t>(nb_max, B - b0);
 		dim3 grid(p.n_tt, p.n_cc, (unsigned)nb);
-		hipLaunchKernelGGL(dense_bwd_f32_fast, grid, dim3(p.threads), p.lds_bytes, st, d_attn + b0 * T * T * H,
-		                   q + b0 * T * HW, k + b0 * T * HW, dq + b0 * T * HW, dkp, (int)T, (int)H, (int)W, scale);
+		launch_bwd_fast(p, grid, st, d_attn + b0 * T * T * H, q + b0 * T * HW, k + b0 * T * HW, dq + b0 * T * HW, dkp,
+		                (int)T, (int)H, (int)W, scale);
 		L1_LAUNCH_CHECK();
 		const int64_t ne = nb * T * HW;
 		const bool vec = ((T * HW) % 4 == 0) && ((((uintptr_t)dkp) | ((uintptr_t)dk)) & 15) == 0;
