@@ -255,9 +255,7 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 // fp32 backward, fast path
 // ------------------------------------------------------------------------------------------
 
-constexpr int BWD_TT = 32;          // dst tokens per workgroup (register-resident q and dq)
-constexpr int BWD_SJ = 4;           // src tokens per staging step
-constexpr int BWD_TTP = BWD_TT + 4; // LDS row pitch: keeps 16-byte alignment for ds_read_b128
+constexpr int BWD_SJ = 4;  // src tokens per staging step
 constexpr float BWD_PRESCALE = 18446744073709551616.0f;  // 2^64
 
 // sign(x) for pre-scaled differences: x is (q-k)*2^64, so every non-zero difference of
@@ -291,53 +289,67 @@ __device__ __forceinline__ void pair_step4(const float* qc, float kc, const floa
 	    : "v"(qc[0]), "v"(qc[1]), "v"(qc[2]), "v"(qc[3]), "v"(kc), "v"(g.x), "v"(g.y), "v"(g.z), "v"(g.w));
 }
 
-// grid.x = dst tiles, grid.y = column chunks of blockDim.x, grid.z = batches of this launch.
+// grid.x = dst tiles of tt_rows tokens, grid.y = column chunks of blockDim.x, grid.z = batches.
 // dkp: [n_ttiles][nb][T][HW] partials (or dk itself when there is a single dst tile).
-// PER = staged dA values per thread and step (ceil(BWD_SJ*BWD_TT*H / blockDim.x) <= PER).  The dA and
-// k values of step n+1 are fetched into registers before the math of step n, so their latency is
-// covered by a whole step of VALU work.
-template <int PER>
-__global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restrict__ dA, const float* __restrict__ q,
-                                                             const float* __restrict__ k, float* __restrict__ dq,
-                                                             float* __restrict__ dkp, int Tn, int H, int W, float scale)
+//
+// TT = dst tokens per workgroup: a lane keeps TT pre-scaled q values and TT dq sums in registers.
+// Two families: TT 32 with up to 1024 threads (4 waves per SIMD), and TT 64..88 with up to 512
+// threads (2 waves per SIMD, 256 registers each), which cuts the number of dk partials up to
+// threefold; the host picks the TT that fills the chip most evenly.
+// The workgroup stages dA only for the heads its columns belong to.
+// PER = staged dA values per thread and step (ceil(BWD_SJ*tt_rows*heads / blockDim.x) <= PER).  The dA
+// and k values of step n+1 are fetched into registers before the math of step n, so their latency
+// is covered by a whole step of VALU work.
+template <int TT, int MAXTHREADS, int PER>
+__global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __restrict__ dA,
+                                                                   const float* __restrict__ q,
+                                                                   const float* __restrict__ k,
+                                                                   float* __restrict__ dq, float* __restrict__ dkp,
+                                                                   int Tn, int H, int W, float scale)
 {
-	extern __shared__ float gl[];  // [BWD_SJ][H][BWD_TTP]
+	constexpr int TTP = TT + 4;  // LDS row pitch: keeps 16-byte alignment for ds_read_b128
+	constexpr int tt_rows = TT;
+	extern __shared__ float gl[];   // [BWD_SJ][HB][TTP]
 	const unsigned HW = (unsigned)(H * W);
-	const unsigned col_raw = blockIdx.y * blockDim.x + threadIdx.x;
-	// lanes past the last column shadow column 0: same inputs, same arithmetic, and they store
-	// the same bits to the same addresses as the lane that owns column 0
-	const unsigned col = col_raw < HW ? col_raw : 0u;
-	const int h = (int)(col / (unsigned)W);
+	const unsigned col0 = blockIdx.y * blockDim.x;
+	const unsigned col_raw = col0 + threadIdx.x;
+	// lanes past the last column shadow the chunk's first column: same inputs, same arithmetic, and
+	// they store the same bits to the same addresses as the lane that owns that column
+	const unsigned col = col_raw < HW ? col_raw : col0;
+	const int h_lo = (int)(col0 / (unsigned)W);
+	const unsigned col_end = min(HW, col0 + blockDim.x) - 1u;
+	const int HB = (int)(col_end / (unsigned)W) - h_lo + 1;  // heads this workgroup touches
+	const int hl = (int)(col / (unsigned)W) - h_lo;
 	const int b = blockIdx.z, nb = gridDim.z;
-	const int tt = blockIdx.x, t0 = tt * BWD_TT;
+	const int tt = blockIdx.x, t0 = tt * tt_rows;
 	// wave-uniform row bases; lanes add the 32-bit column
 	const float* const q_b = q + (int64_t)b * Tn * HW;
 	const float* const k_b = k + (int64_t)b * Tn * HW;
-	const float* const dA_b = dA + ((int64_t)b * Tn * Tn + t0) * H;
+	const float* const dA_b = dA + ((int64_t)b * Tn * Tn + t0) * H + h_lo;
 	float* const dkp_b = dkp + ((int64_t)tt * nb + b) * Tn * HW;
 
-	float qc[BWD_TT], dqa[BWD_TT];
+	float qc[TT], dqa[TT];
 #pragma unroll
-	for (int i = 0; i < BWD_TT; i++) {
+	for (int i = 0; i < TT; i++) {
 		const int t = min(t0 + i, Tn - 1);
 		qc[i] = (q_b + (int64_t)t * HW)[col] * BWD_PRESCALE;
 		dqa[i] = 0.0f;
 	}
 
 	// staging roles of this thread: element e = threadIdx.x + r*blockDim.x of the [j][i][hh] step tile
-	const int n_stage = BWD_SJ * BWD_TT * H;
+	const int n_stage = BWD_SJ * tt_rows * HB;
 	int st_j[PER], st_lds[PER];
 	int64_t st_off[PER];
 	bool st_ok[PER];
 #pragma unroll
 	for (int r = 0; r < PER; r++) {
 		const int e = threadIdx.x + r * blockDim.x;
-		const int j = e / (BWD_TT * H), rr = e % (BWD_TT * H);
-		const int i = rr / H, hh = rr % H;
+		const int j = e / (tt_rows * HB), rr = e % (tt_rows * HB);
+		const int i = rr / HB, hh = rr % HB;
 		st_j[r] = j;
 		st_ok[r] = e < n_stage && t0 + i < Tn;
-		st_off[r] = (int64_t)j * Tn * H + rr;
-		st_lds[r] = e < n_stage ? (j * H + hh) * BWD_TTP + i : -1;
+		st_off[r] = ((int64_t)j * Tn + i) * H + hh;
+		st_lds[r] = e < n_stage ? (j * HB + hh) * TTP + i : -1;
 	}
 	float g_pre[PER], k_pre[BWD_SJ];
 	auto prefetch = [&](int s0) {
@@ -366,16 +378,16 @@ __global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restri
 		if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
 		{
 			// all dA values of this step for the lane's head, read one float4 ahead of their use
-			const float4* gp0 = reinterpret_cast<const float4*>(gl + h * BWD_TTP);
-			constexpr int NI4 = BWD_TT / 4;
+			const float4* gp0 = reinterpret_cast<const float4*>(gl + hl * TTP);
+			constexpr int NI4 = TT / 4;
 			float4 g_cur = gp0[0];
 #pragma unroll
 			for (int j = 0; j < BWD_SJ; j++) {
 #pragma unroll
 				for (int i4 = 0; i4 < NI4; i4++) {
 					float4 g_nxt = g_cur;
-					if (i4 + 1 < NI4) g_nxt = gp0[(j * H * BWD_TTP) / 4 + i4 + 1];
-					else if (j + 1 < BWD_SJ) g_nxt = gp0[((j + 1) * H * BWD_TTP) / 4];
+					if (i4 + 1 < NI4) g_nxt = gp0[(j * HB * TTP) / 4 + i4 + 1];
+					else if (j + 1 < BWD_SJ) g_nxt = gp0[((j + 1) * HB * TTP) / 4];
 					__builtin_amdgcn_sched_barrier(0);
 					pair_step4(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
 					g_cur = g_nxt;
@@ -392,7 +404,7 @@ __global__ __launch_bounds__(1024) void dense_bwd_f32_fast(const float* __restri
 	}
 	float* const dq_b = dq + (int64_t)b * Tn * HW;
 #pragma unroll
-	for (int i = 0; i < BWD_TT; i++) {
+	for (int i = 0; i < TT; i++) {
 		const int t = t0 + i;
 		if (t < Tn) (dq_b + (int64_t)t * HW)[col] = dqa[i] * scale;
 	}
@@ -498,24 +510,40 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 
 struct BwdPlan {
 	bool fast;
-	int threads, n_cc, n_tt, per;
+	bool wide;        // TTMAX 96 / 512-thread instantiation
+	int threads, n_cc, n_tt, tt_rows, per;
 	size_t lds_bytes;
 	size_t per_batch_bytes;  // partial-dk scratch for one batch (0 when a single dst tile)
 };
+
+constexpr int N_CU = 256;
 
 BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 {
 	BwdPlan p{};
 	const int64_t HW = H * W;
-	p.lds_bytes = (size_t)BWD_SJ * H * BWD_TTP * sizeof(float);
-	p.fast = B >= 1 && T >= 16 && HW >= 32 && p.lds_bytes <= 64 * 1024 && T <= (1 << 30) && B <= 65535 &&
-	         HW <= (int64_t)1024 * 65535;
+	p.fast = B >= 1 && T >= 16 && HW >= 32 && T <= (1 << 30) && B <= 65535 && HW <= (int64_t)512 * 65535;
 	if (!p.fast) return p;
-	p.threads = (int)std::min<int64_t>(1024, l1_cdiv(HW, 64) * 64);
+	// wide tiles pay off once there are enough dst tokens to give every CU a few workgroups
+	p.wide = T >= 1024 && B * l1_cdiv(HW, 512) * l1_cdiv(T, 88) >= N_CU;
+	const int maxthreads = p.wide ? 512 : 1024;
+	p.threads = (int)std::min<int64_t>(maxthreads, l1_cdiv(HW, 64) * 64);
 	p.n_cc = (int)l1_cdiv(HW, p.threads);
-	p.n_tt = (int)l1_cdiv(T, BWD_TT);
-	p.per = (int)l1_cdiv((int64_t)BWD_SJ * BWD_TT * H, p.threads);
-	if (p.per > 16) { p.fast = false; return p; }
+	p.tt_rows = p.wide ? 88 : 32;
+	if (p.wide) {
+		// one workgroup per CU at a time: pick the tile height that wastes the least of the last round
+		double best = 1e30;
+		for (int tr = 64; tr <= 88; tr += 8) {
+			const int64_t wgs = B * p.n_cc * l1_cdiv(T, tr);
+			const double cost = (double)l1_cdiv(wgs, N_CU) * tr * (1.0 + 3.0 / tr);  // rounds x rows, plus partial traffic
+			if (cost < best) { best = cost; p.tt_rows = tr; }
+		}
+	}
+	p.n_tt = (int)l1_cdiv(T, p.tt_rows);
+	const int64_t hb_max = std::min<int64_t>(H, (p.threads + W - 2) / W + 1);
+	p.lds_bytes = (size_t)BWD_SJ * hb_max * (p.tt_rows + 4) * sizeof(float);
+	p.per = (int)l1_cdiv((int64_t)BWD_SJ * p.tt_rows * hb_max, p.threads);
+	if (p.lds_bytes > 64 * 1024 || p.per > 16 || (p.wide && p.per > 8)) { p.fast = false; return p; }
 	p.per_batch_bytes = p.n_tt > 1 ? (size_t)p.n_tt * T * HW * sizeof(float) : 0;
 	return p;
 }
@@ -523,14 +551,23 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* dA, const float* q, const float* k,
                      float* dq, float* dkp, int T, int H, int W, float scale)
 {
-#define L1_BWD_CASE(PERV)                                                                                       \
-	hipLaunchKernelGGL(dense_bwd_f32_fast<PERV>, grid, dim3(p.threads), p.lds_bytes, st, dA, q, k, dq, dkp, T, H, W, \
-	                   scale)
-	if (p.per <= 1) L1_BWD_CASE(1);
-	else if (p.per <= 2) L1_BWD_CASE(2);
-	else if (p.per <= 4) L1_BWD_CASE(4);
-	else if (p.per <= 8) L1_BWD_CASE(8);
-	else L1_BWD_CASE(16);
+#define L1_BWD_CASE(TTV, MT, PERV)                                                                              \
+	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV>), grid, dim3(p.threads), p.lds_bytes, st, dA, q, k, dq,   \
+	                   dkp, T, H, W, scale)
+	if (p.wide) {
+		switch (p.tt_rows) {
+		case 64: L1_BWD_CASE(64, 512, 8); break;
+		case 72: L1_BWD_CASE(72, 512, 8); break;
+		case 80: L1_BWD_CASE(80, 512, 8); break;
+		default: L1_BWD_CASE(88, 512, 8); break;
+		}
+	} else {
+		if (p.per <= 1) L1_BWD_CASE(32, 1024, 1);
+		else if (p.per <= 2) L1_BWD_CASE(32, 1024, 2);
+		else if (p.per <= 4) L1_BWD_CASE(32, 1024, 4);
+		else if (p.per <= 8) L1_BWD_CASE(32, 1024, 8);
+		else L1_BWD_CASE(32, 1024, 16);
+	}
 #undef L1_BWD_CASE
 }
 
