@@ -94,6 +94,24 @@ __global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict_
 
 constexpr int FWD_SJ = 8;  // src rows finished between two output flushes
 
+// Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.
+// This maps the flat dispatch index to a logical one such that logically consecutive workgroups
+// (which share k rows) land on the same XCD: XCD x runs the logical range [x*n/8, (x+1)*n/8).
+struct LogicalBlock { int x, y, z; };
+__device__ __forceinline__ LogicalBlock xcd_remap()
+{
+	const unsigned nx = gridDim.x, ny = gridDim.y, n = nx * ny * gridDim.z;
+	const unsigned flat = blockIdx.x + nx * (blockIdx.y + ny * blockIdx.z);
+	const unsigned per = n / 8u;
+	unsigned m = flat;
+	if (flat < per * 8u) m = (flat % 8u) * per + flat / 8u;
+	LogicalBlock lb;
+	lb.x = (int)(m % nx);
+	lb.y = (int)((m / nx) % ny);
+	lb.z = (int)(m / (nx * ny));
+	return lb;
+}
+
 // grid.x = dst tiles of 64 tokens, grid.y = src chunks, grid.z = B * head groups.
 // block = 64 * NW threads, NW = heads per group (<= 16); wave w of the block owns head hg*NW + w.
 // W is a compile-time multiple of 16; q and k must be 16-byte aligned.
@@ -106,9 +124,10 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const int NW = blockDim.x >> 6;
-	const int b = blockIdx.z / n_hg, hg = blockIdx.z % n_hg;
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.z / n_hg, hg = lb.z % n_hg;
 	const int h = min(hg * NW + wave, H - 1);  // surplus waves of the last group redo head H-1, never stored
-	const int t0 = blockIdx.x * WAVE;
+	const int t0 = lb.x * WAVE;
 	const int t = min(t0 + lane, Tn - 1);
 
 	float qr[W];
@@ -127,7 +146,7 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (t0 + o_tl)) * H + hg * NW + o_hh;
 	const int64_t o_pitch = (int64_t)Tn * H;
 
-	const int s_begin = blockIdx.y * s_chunk;
+	const int s_begin = lb.y * s_chunk;
 	const int s_end = min(Tn, s_begin + s_chunk);
 	for (int s0 = s_begin; s0 < s_end; s0 += FWD_SJ) {
 #pragma unroll
@@ -177,9 +196,10 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const int NW = blockDim.x >> 6;
-	const int b = blockIdx.z / n_hg, hg = blockIdx.z % n_hg;
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.z / n_hg, hg = lb.z % n_hg;
 	const int h = min(hg * NW + wave, H - 1);
-	const int t0 = blockIdx.x * WAVE;
+	const int t0 = lb.x * WAVE;
 	const int t = min(t0 + lane, Tn - 1);
 
 	float qr[W];
@@ -204,7 +224,7 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 	// of the tensor (computed but never stored) read valid memory
 	const float* const k_last = kb + (int64_t)(Tn - 1) * krow + (CPR - 1) * 32;
 
-	const int s_begin = blockIdx.y * s_chunk;
+	const int s_begin = lb.y * s_chunk;
 	const int s_end = min(Tn, s_begin + s_chunk);
 	f32x16 b0l, b0h, b1l, b1h;
 	const float* kp = kb + (int64_t)s_begin * krow;  // chunk being prefetched
