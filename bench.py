@@ -23,12 +23,14 @@ for _p in (ROOT, os.path.join(ROOT, "l1-attention_amd"), os.path.join(ROOT, "tes
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-P_VALU_TOPS = 78.6     # 256 CU x 4 SIMD x 16 lanes x 2 (packed fp32) x 2.4 GHz; the 157.3 TFLOP/s figure counts FMA as 2
+P_VALU_TOPS = 78.6     # 256 CU x 4 SIMD x 32 fp32 lanes/clk x 2.4 GHz; the 157.3 TFLOP/s datasheet figure counts FMA as 2
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
-# HBM bytes per dense-backward launch (B=8,T=4096,H=16,W=64) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-# scaled by a copy kernel of known size; None until measured (see profiles/).
-DENSE_BWD_TRAFFIC_BYTES = None
+# HBM bytes per dense-backward launch (B=8,T=4096,H=16,W=64) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/dense_B8_T4096_H16_W64_pmc_*.txt), scaled by what three 1 GiB device copies read on the same
+# counters (profiles/copy_1GiB_pmc_*.txt: FETCH_SIZE 0.5 per KiB -> x2.0, WRITE_SIZE 1.0 per KiB -> x1.0):
+# main kernel 4925279*2 + 8519680 KiB, dk reduce 4194587*2 + 131072 KiB.
+DENSE_BWD_TRAFFIC_BYTES = (4925279 * 2 + 8519680 + 4194587 * 2 + 131072) * 1024
 
 
 def log(*a):
@@ -256,8 +258,8 @@ def main():
         "traffic": DENSE_BWD_TRAFFIC_BYTES,
         "flops_per_launch": 4 * N, "avg_launch_ms": d["bwd_ms"],
         "note": "algorithmic ops (4 per pair-element) over the HIP-event time of the backward launch; "
-                "peak = packed-fp32 VALU issue rate, which this library does not use "
-                "(scalar-per-lane fp32 peaks at 39.3)",
+                "peak = nominal fp32 VALU issue rate (one wave64 instruction per SIMD every 2 cycles at "
+                "2.4 GHz); traffic = HBM bytes of the launch against 8.5 GiB algorithmic (dA once + q,k,dq,dk)",
     }
     out = {
         "metric": "dense fwd+bwd GOP/s & % fp32 VALU peak; sparse fwd+bwd edges/s & HBM GB/s",
