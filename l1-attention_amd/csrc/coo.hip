@@ -29,7 +29,7 @@ constexpr int RS_BITS = 8;
 constexpr int RS_DIGITS = 1 << RS_BITS;
 
 // stats words written by the extract kernels
-enum { ST_MAXKEY = 0, ST_BAD = 1, ST_MAXDEG_DST = 2, ST_MAXDEG_SRC = 3, ST_WORDS = 4 };
+enum { ST_MAXKEY = 0, ST_BAD = 1, ST_MAXDEG_DST = 2, ST_MAXDEG_SRC = 3, ST_NLONG_DST = 4, ST_NLONG_SRC = 5, ST_WORDS = 8 };
 
 template <typename IdxT>
 __global__ __launch_bounds__(256) void coo_extract(const IdxT* __restrict__ co, int64_t stride, int64_t E,
@@ -204,11 +204,16 @@ __global__ __launch_bounds__(256) void plan_fill_csc(const int* __restrict__ row
 	csc_slot[i] = slot_of_row[row];
 }
 
-// longest segment of a pointer array with n_keys segments
-__global__ __launch_bounds__(256) void max_segment(const int* __restrict__ ptr, int n_keys, int* __restrict__ out)
+// longest segment of a pointer array with n_keys segments, and the list of keys whose segment is
+// longer than PLAN_LONG_SEGMENT (list order is arbitrary: every entry is processed independently)
+__global__ __launch_bounds__(256) void max_segment(const int* __restrict__ ptr, int n_keys, int* __restrict__ out,
+                                                     int* __restrict__ long_list, int* __restrict__ n_long)
 {
 	const int key = blockIdx.x * 256 + threadIdx.x;
-	if (key < n_keys) atomicMax(out, ptr[key + 1] - ptr[key]);
+	if (key >= n_keys) return;
+	const int deg = ptr[key + 1] - ptr[key];
+	atomicMax(out, deg);
+	if (deg > PLAN_LONG_SEGMENT) long_list[atomicAdd(n_long, 1)] = key;
 }
 
 __global__ void fill_words(int* __restrict__ a, int n, int v)
@@ -228,6 +233,8 @@ __global__ void plan_header(int* __restrict__ hdr, int E, int T, const int* __re
 		hdr[PLAN_H_MAXDEG_DST] = stats[ST_MAXDEG_DST];
 		hdr[PLAN_H_MAXDEG_SRC] = stats[ST_MAXDEG_SRC];
 		hdr[PLAN_H_E_VALID] = dst_ptr[T];  // rows with the sentinel key T sort behind this position
+		hdr[PLAN_H_NLONG_DST] = stats[ST_NLONG_DST];
+		hdr[PLAN_H_NLONG_SRC] = stats[ST_NLONG_SRC];
 	}
 }
 
@@ -414,14 +421,14 @@ int l1attn_sparse_plan_build(const int32_t* coo, int64_t coo_stride, int64_t E, 
 	                   words + L.csr_row, slot_of_row);
 	L1_LAUNCH_CHECK();
 	if (T > 0) hipLaunchKernelGGL(max_segment, dim3((unsigned)l1_cdiv(T, 256)), dim3(256), 0, st, words + L.dst_ptr,
-	                              (int)T, stats + ST_MAXDEG_DST);
+	                              (int)T, stats + ST_MAXDEG_DST, words + L.long_dst, stats + ST_NLONG_DST);
 	L1_LAUNCH_CHECK();
 	rc = sort_rows_by_key(src32, E, bits, sb, st, &ks, &rs);
 	if (rc) return rc;
 	hipLaunchKernelGGL(segment_ptrs, dim3(gptr), dim3(256), 0, st, ks, (int)E, (int)(T + 2), words + L.src_ptr);
 	L1_LAUNCH_CHECK();
 	if (T > 0) hipLaunchKernelGGL(max_segment, dim3((unsigned)l1_cdiv(T, 256)), dim3(256), 0, st, words + L.src_ptr,
-	                              (int)T, stats + ST_MAXDEG_SRC);
+	                              (int)T, stats + ST_MAXDEG_SRC, words + L.long_src, stats + ST_NLONG_SRC);
 	L1_LAUNCH_CHECK();
 	hipLaunchKernelGGL(plan_fill_csc, dim3(g256), dim3(256), 0, st, rs, dst32, slot_of_row, (int)E,
 	                   words + L.csc_dst, words + L.csc_slot);

@@ -12,9 +12,13 @@ enum {
 	PLAN_H_MAXDEG_DST = 4,  // longest dst segment
 	PLAN_H_MAXDEG_SRC = 5,  // longest src segment
 	PLAN_H_E_VALID = 6,     // rows kept
+	PLAN_H_NLONG_DST = 7,   // dst tokens with more than PLAN_LONG_SEGMENT edges (entries of long_dst)
+	PLAN_H_NLONG_SRC = 8,   // same for src tokens
 	PLAN_H_WORDS = 16
 };
-constexpr int PLAN_MAGIC = 0x4c314131;  // "L1A1"
+constexpr int PLAN_MAGIC = 0x4c314132;  // "L1A2"
+// Segments longer than this are walked by a whole workgroup instead of one wavefront.
+constexpr int PLAN_LONG_SEGMENT = 128;
 
 struct PlanLayout {
 	// offsets in int32 words from the start of the plan
@@ -24,6 +28,9 @@ struct PlanLayout {
 	size_t csr_row;   // [E]    original row of each slot
 	size_t csc_dst;   // [E]    dst token of each src-sorted entry
 	size_t csc_slot;  // [E]    dst-sorted slot of each src-sorted entry
+	size_t long_dst;  // [long_cap] dst tokens whose segment is longer than PLAN_LONG_SEGMENT (any order)
+	size_t long_src;  // [long_cap]
+	size_t long_cap;  // E / PLAN_LONG_SEGMENT + 1: no edge list has more long segments than that
 	size_t total_bytes;
 };
 
@@ -38,6 +45,10 @@ static inline PlanLayout plan_layout(int64_t E, int64_t T)
 	L.csr_row = w; w += ea;
 	L.csc_dst = w; w += ea;
 	L.csc_slot = w; w += ea;
+	L.long_cap = (size_t)(E > 0 ? E : 0) / PLAN_LONG_SEGMENT + 1;
+	const size_t la = l1_align_up(L.long_cap, 64);
+	L.long_dst = w; w += la;
+	L.long_src = w; w += la;
 	L.total_bytes = w * 4;
 	return L;
 }

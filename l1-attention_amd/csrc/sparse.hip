@@ -69,40 +69,94 @@ template <typename T> __device__ __forceinline__ T sgn_t(T x) { return (T)((x > 
 // geometry of one work item, shared by all kernels
 struct Geo {
 	int Tn, H, W, Wv, E;
-	int log2G;  // lanes per head = 1 << log2G
-	int n_hc;   // head chunks per token = ceil(H / (64 >> log2G))
+	int log2G;     // lanes per head = 1 << log2G
+	int n_hc;      // head chunks per token = ceil(H / (64 >> log2G))
+	int long_on;   // 1: segments longer than PLAN_LONG_SEGMENT are left to the workgroup-per-segment launch
 };
 
 struct Lane {
 	int tok, h, sub;
 	bool head_ok;
+	int pb, pe;    // this wave's share [pb, pe) of the segment
+	int p0, p1;    // the whole segment
+	int wave;
 };
 
-__device__ __forceinline__ bool wave_item(const Geo& g, Lane& L)
+// Work decomposition.
+//  NWV == 1: wave-per-item launch.  grid.x covers the Tn*n_hc (token, head chunk) items, four per block;
+//            grid.y = batch.  Items whose segment is "long" are skipped when g.long_on.
+//  NWV  > 1: workgroup-per-item launch over the plan's list of long tokens.  grid.x = capacity of the
+//            list (entries beyond the count on the device exit at once), grid.y = batch, grid.z = head
+//            chunk; the NWV waves take contiguous, equal shares of the segment in wave order.
+template <int NWV>
+__device__ __forceinline__ bool wave_item(const Geo& g, const int* __restrict__ ptr, const int* __restrict__ long_list,
+                                          const int* __restrict__ n_long, Lane& L)
 {
 	const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 	const int lane = threadIdx.x & 63;
-	const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
-	if (item >= (int64_t)g.Tn * g.n_hc) return false;
-	L.tok = (int)(item / g.n_hc);
-	const int hc = (int)(item % g.n_hc);
+	int hc;
+	if (NWV == 1) {
+		const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
+		if (item >= (int64_t)g.Tn * g.n_hc) return false;
+		L.tok = (int)(item / g.n_hc);
+		hc = (int)(item % g.n_hc);
+	} else {
+		if ((int)blockIdx.x >= *n_long) return false;  // uniform over the workgroup
+		L.tok = long_list[blockIdx.x];
+		hc = blockIdx.z;
+	}
+	L.p0 = ptr[L.tok];
+	L.p1 = ptr[L.tok + 1];
+	const int deg = L.p1 - L.p0;
+	if (NWV == 1) {
+		if (g.long_on && deg > PLAN_LONG_SEGMENT) return false;
+		L.pb = L.p0;
+		L.pe = L.p1;
+	} else {
+		const int share = (deg + NWV - 1) / NWV;
+		L.pb = min(L.p1, L.p0 + wave * share);
+		L.pe = min(L.p1, L.pb + share);
+	}
+	L.wave = wave;
 	L.sub = lane & ((1 << g.log2G) - 1);
 	L.h = hc * (64 >> g.log2G) + (lane >> g.log2G);
 	L.head_ok = L.h < g.H;
 	return true;
 }
 
+// Sum of x over the NWV waves of the workgroup, in wave order (bitwise reproducible), returned to
+// every wave.  smem: NWV*64 elements per call site; the caller separates uses with the barriers here.
+template <typename T, int NWV>
+__device__ __forceinline__ T wg_sum(T x, T* smem, int wave)
+{
+	if (NWV == 1) return x;
+	const int lane = threadIdx.x & 63;
+	__syncthreads();
+	smem[wave * 64 + lane] = x;
+	__syncthreads();
+	T s = smem[lane];
+#pragma unroll
+	for (int w = 1; w < NWV; w++) s += smem[w * 64 + lane];
+	return s;
+}
+
+// edges in flight per wave: rows of EU edges are requested before the first is used
+template <int MC> struct Unroll { static constexpr int EU = MC == 1 ? 4 : 1; };
+
 // ---------------------------------------------------------------------------------- forward
 
 // dst pass: logits, softmax with the "+1" denominator, value sum.  Writes vo rows and P.
-template <typename T, int VEC, int MC>
-__global__ __launch_bounds__(256) void sparse_fwd_dst(const T* __restrict__ v, const T* __restrict__ q,
-                                                        const T* __restrict__ k, const int* __restrict__ dst_ptr,
-                                                        const int* __restrict__ csr_src, T* __restrict__ vo,
-                                                        T* __restrict__ P, Geo g, int use_softmax, T scale)
+template <typename T, int VEC, int MC, int NWV>
+__global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_dst(
+    const T* __restrict__ v, const T* __restrict__ q, const T* __restrict__ k, const int* __restrict__ dst_ptr,
+    const int* __restrict__ csr_src, const int* __restrict__ long_list, const int* __restrict__ n_long,
+    T* __restrict__ vo, T* __restrict__ P, Geo g, int use_softmax, T scale)
 {
+	extern __shared__ unsigned char smem_raw[];
+	T* smem = reinterpret_cast<T*>(smem_raw);
+	constexpr int EU = Unroll<MC>::EU;
 	Lane L;
-	if (!wave_item(g, L)) return;
+	if (!wave_item<NWV>(g, dst_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowq = (int64_t)g.H * g.W, rowv = (int64_t)g.H * g.Wv;
 	const T* qb = q + (int64_t)b * g.Tn * rowq;
@@ -112,101 +166,158 @@ __global__ __launch_bounds__(256) void sparse_fwd_dst(const T* __restrict__ v, c
 
 	T qv[MC][VEC], acc[MC][VEC];
 	bool okq[MC], okv[MC];
+	int offq[MC], offv[MC];
 #pragma unroll
 	for (int m = 0; m < MC; m++) {
 		const int w0 = (m * G + L.sub) * VEC;
 		okq[m] = L.head_ok && w0 < g.W;
 		okv[m] = L.head_ok && w0 < g.Wv;
+		offq[m] = L.h * g.W + w0;
+		offv[m] = L.h * g.Wv + w0;
 #pragma unroll
 		for (int i = 0; i < VEC; i++) { qv[m][i] = 0; acc[m][i] = 0; }
-		if (okq[m]) ldv<T, VEC>(qb + (int64_t)L.tok * rowq + L.h * g.W + w0, qv[m]);
+		if (okq[m]) ldv<T, VEC>(qb + (int64_t)L.tok * rowq + offq[m], qv[m]);
 	}
-	const int p0 = dst_ptr[L.tok], p1 = dst_ptr[L.tok + 1];
-	T den = use_softmax ? (T)1 : (T)0;
-	for (int p = p0; p < p1; p++) {
-		const int src = csr_src[p];
-		T d = 0;
-		T vv[MC][VEC];
+	T den = 0;
+	int sidx[EU];
+#pragma unroll
+	for (int u = 0; u < EU; u++) sidx[u] = L.pb < L.pe ? csr_src[min(L.pb + u, L.pe - 1)] : 0;
+	for (int p = L.pb; p < L.pe; p += EU) {
+		T kv[EU][MC][VEC], vv[EU][MC][VEC];
+#pragma unroll
+		for (int u = 0; u < EU; u++)
+#pragma unroll
+			for (int m = 0; m < MC; m++) {
+#pragma unroll
+				for (int i = 0; i < VEC; i++) { kv[u][m][i] = qv[m][i]; vv[u][m][i] = 0; }
+				if (okq[m]) ldv<T, VEC>(kb + (int64_t)sidx[u] * rowq + offq[m], kv[u][m]);
+				if (okv[m]) ldv<T, VEC>(vb + (int64_t)sidx[u] * rowv + offv[m], vv[u][m]);
+			}
+		// indices of the next group, clamped into this wave's share
+#pragma unroll
+		for (int u = 0; u < EU; u++) sidx[u] = csr_src[min(p + EU + u, L.pe - 1)];
+		T d[EU];
+#pragma unroll
+		for (int u = 0; u < EU; u++) {
+			d[u] = 0;
+#pragma unroll
+			for (int m = 0; m < MC; m++)
+#pragma unroll
+				for (int i = 0; i < VEC; i++) d[u] += abs_t(qv[m][i] - kv[u][m][i]);
+		}
+#pragma unroll
+		for (int u = 0; u < EU; u++) d[u] = group_sum(d[u], G);
+#pragma unroll
+		for (int u = 0; u < EU; u++) {
+			if (p + u < L.pe) {  // uniform
+				const T e = exp_t(d[u] * scale);
+				den += e;
+#pragma unroll
+				for (int m = 0; m < MC; m++)
+#pragma unroll
+					for (int i = 0; i < VEC; i++) acc[m][i] += e * vv[u][m][i];
+				if (L.sub == 0 && L.head_ok) Pb[(int64_t)(p + u) * g.H + L.h] = e;
+			}
+		}
+	}
+	// combine the waves of a long segment in wave order
+	den = wg_sum<T, NWV>(den, smem, L.wave);
+#pragma unroll
+	for (int m = 0; m < MC; m++)
+#pragma unroll
+		for (int i = 0; i < VEC; i++) acc[m][i] = wg_sum<T, NWV>(acc[m][i], smem, L.wave);
+	if (use_softmax) den += (T)1;
+	const T inv = use_softmax ? (T)1 / den : (T)1;
+	if (L.wave == 0 || NWV == 1) {
 #pragma unroll
 		for (int m = 0; m < MC; m++) {
-			const int w0 = (m * G + L.sub) * VEC;
-			T kv[VEC];
 #pragma unroll
-			for (int i = 0; i < VEC; i++) { kv[i] = qv[m][i]; vv[m][i] = 0; }
-			if (okq[m]) ldv<T, VEC>(kb + (int64_t)src * rowq + L.h * g.W + w0, kv);
-			if (okv[m]) ldv<T, VEC>(vb + (int64_t)src * rowv + L.h * g.Wv + w0, vv[m]);
-#pragma unroll
-			for (int i = 0; i < VEC; i++) d += abs_t(qv[m][i] - kv[i]);
+			for (int i = 0; i < VEC; i++) acc[m][i] *= inv;
+			if (okv[m]) stv<T, VEC>(vo + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m], acc[m]);
 		}
-		d = group_sum(d, G);
-		const T e = exp_t(d * scale);
-		den += e;
-#pragma unroll
-		for (int m = 0; m < MC; m++)
-#pragma unroll
-			for (int i = 0; i < VEC; i++) acc[m][i] += e * vv[m][i];
-		if (L.sub == 0 && L.head_ok) Pb[(int64_t)p * g.H + L.h] = e;
-	}
-	const T inv = use_softmax ? (T)1 / den : (T)1;
-#pragma unroll
-	for (int m = 0; m < MC; m++) {
-		const int w0 = (m * G + L.sub) * VEC;
-#pragma unroll
-		for (int i = 0; i < VEC; i++) acc[m][i] *= inv;
-		if (okv[m]) stv<T, VEC>(vo + ((int64_t)b * g.Tn + L.tok) * rowv + L.h * g.Wv + w0, acc[m]);
 	}
 	// the weights below were stored by lane 0 of each head group: make them visible to its other lanes
 	__threadfence();
 	if (use_softmax && L.head_ok) {
-		// normalise the stored weights; the G lanes of a head take every G-th slot
-		for (int p = p0 + L.sub; p < p1; p += G) Pb[(int64_t)p * g.H + L.h] *= inv;
+		// normalise the stored weights of this wave's share; the G lanes of a head take every G-th slot
+		for (int p = L.pb + L.sub; p < L.pe; p += G) Pb[(int64_t)p * g.H + L.h] *= inv;
 	}
 }
 
 // bidi src pass: vo[b,src] += sum over the src's edges of p * vb[b,dst]   (cpp/l1attn_sparse_bidi_drv.cpp:93-96)
-template <typename T, int VEC, int MC>
-__global__ __launch_bounds__(256) void sparse_fwd_src(const T* __restrict__ vbk, const int* __restrict__ src_ptr,
-                                                        const int* __restrict__ csc_dst,
-                                                        const int* __restrict__ csc_slot, const T* __restrict__ P,
-                                                        T* __restrict__ vo, Geo g)
+template <typename T, int VEC, int MC, int NWV>
+__global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_src(
+    const T* __restrict__ vbk, const int* __restrict__ src_ptr, const int* __restrict__ csc_dst,
+    const int* __restrict__ csc_slot, const int* __restrict__ long_list, const int* __restrict__ n_long,
+    const T* __restrict__ P, T* __restrict__ vo, Geo g)
 {
+	extern __shared__ unsigned char smem_raw[];
+	T* smem = reinterpret_cast<T*>(smem_raw);
+	constexpr int EU = Unroll<MC>::EU;
 	Lane L;
-	if (!wave_item(g, L)) return;
+	if (!wave_item<NWV>(g, src_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowv = (int64_t)g.H * g.Wv;
 	const T* vb = vbk + (int64_t)b * g.Tn * rowv;
 	const T* Pb = P + (int64_t)b * g.E * g.H;
 	T acc[MC][VEC];
 	bool okv[MC];
+	int offv[MC];
 #pragma unroll
 	for (int m = 0; m < MC; m++) {
 		okv[m] = L.head_ok && (m * G + L.sub) * VEC < g.Wv;
+		offv[m] = L.h * g.Wv + (m * G + L.sub) * VEC;
 #pragma unroll
 		for (int i = 0; i < VEC; i++) acc[m][i] = 0;
 	}
-	const int i0 = src_ptr[L.tok], i1 = src_ptr[L.tok + 1];
-	for (int e = i0; e < i1; e++) {
-		const int dst = csc_dst[e], slot = csc_slot[e];
-		const T pe = L.head_ok ? Pb[(int64_t)slot * g.H + L.h] : (T)0;
+	int didx[EU], slot[EU];
 #pragma unroll
-		for (int m = 0; m < MC; m++) {
-			T x[VEC];
+	for (int u = 0; u < EU; u++) {
+		const int e = min(L.pb + u, L.pe - 1);
+		didx[u] = L.pb < L.pe ? csc_dst[e] : 0;
+		slot[u] = L.pb < L.pe ? csc_slot[e] : 0;
+	}
+	for (int e0 = L.pb; e0 < L.pe; e0 += EU) {
+		T x[EU][MC][VEC], pe[EU];
 #pragma unroll
-			for (int i = 0; i < VEC; i++) x[i] = 0;
-			if (okv[m]) ldv<T, VEC>(vb + (int64_t)dst * rowv + L.h * g.Wv + (m * G + L.sub) * VEC, x);
+		for (int u = 0; u < EU; u++) {
+			pe[u] = L.head_ok ? Pb[(int64_t)slot[u] * g.H + L.h] : (T)0;
 #pragma unroll
-			for (int i = 0; i < VEC; i++) acc[m][i] += pe * x[i];
+			for (int m = 0; m < MC; m++) {
+#pragma unroll
+				for (int i = 0; i < VEC; i++) x[u][m][i] = 0;
+				if (okv[m]) ldv<T, VEC>(vb + (int64_t)didx[u] * rowv + offv[m], x[u][m]);
+			}
 		}
+#pragma unroll
+		for (int u = 0; u < EU; u++) {
+			const int e = min(e0 + EU + u, L.pe - 1);
+			didx[u] = csc_dst[e];
+			slot[u] = csc_slot[e];
+		}
+#pragma unroll
+		for (int u = 0; u < EU; u++)
+			if (e0 + u < L.pe)
+#pragma unroll
+				for (int m = 0; m < MC; m++)
+#pragma unroll
+					for (int i = 0; i < VEC; i++) acc[m][i] += pe[u] * x[u][m][i];
 	}
 #pragma unroll
-	for (int m = 0; m < MC; m++) {
-		if (okv[m]) {
-			T* o = vo + ((int64_t)b * g.Tn + L.tok) * rowv + L.h * g.Wv + (m * G + L.sub) * VEC;
-			T x[VEC];
-			ldv<T, VEC>(o, x);
+	for (int m = 0; m < MC; m++)
 #pragma unroll
-			for (int i = 0; i < VEC; i++) x[i] += acc[m][i];
-			stv<T, VEC>(o, x);
+		for (int i = 0; i < VEC; i++) acc[m][i] = wg_sum<T, NWV>(acc[m][i], smem, L.wave);
+	if (L.wave == 0 || NWV == 1) {
+#pragma unroll
+		for (int m = 0; m < MC; m++) {
+			if (okv[m]) {
+				T* o = vo + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m];
+				T y[VEC];
+				ldv<T, VEC>(o, y);
+#pragma unroll
+				for (int i = 0; i < VEC; i++) y[i] += acc[m][i];
+				stv<T, VEC>(o, y);
+			}
 		}
 	}
 }
@@ -216,16 +327,18 @@ __global__ __launch_bounds__(256) void sparse_fwd_src(const T* __restrict__ vbk,
 // dst pass.  For every edge of the dst:  dp = v[src].dvo[dst] (+ vb[dst].dvo[src] for bidi);
 // S = sum p*dp;  dq[dst] = scale * sum sign(q-k) * p * (dp - S)  accumulated as X - S*Y in one walk;
 // bidi: dvb[dst] = sum p * dvo[src].  Leaves da = p*(dp - S) (or p*dp) per edge in DA.
-template <typename T, int VEC, int MC, bool BIDI>
-__global__ __launch_bounds__(256) void sparse_bwd_dst(const T* __restrict__ dvo, const T* __restrict__ v,
-                                                        const T* __restrict__ vbk, const T* __restrict__ q,
-                                                        const T* __restrict__ k, const int* __restrict__ dst_ptr,
-                                                        const int* __restrict__ csr_src, const T* __restrict__ P,
-                                                        T* __restrict__ DA, T* __restrict__ dq,
-                                                        T* __restrict__ dvb, Geo g, int use_softmax, T scale)
+template <typename T, int VEC, int MC, bool BIDI, int NWV>
+__global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_dst(
+    const T* __restrict__ dvo, const T* __restrict__ v, const T* __restrict__ vbk, const T* __restrict__ q,
+    const T* __restrict__ k, const int* __restrict__ dst_ptr, const int* __restrict__ csr_src,
+    const int* __restrict__ long_list, const int* __restrict__ n_long, const T* __restrict__ P,
+    T* __restrict__ DA, T* __restrict__ dq, T* __restrict__ dvb, Geo g, int use_softmax, T scale)
 {
+	extern __shared__ unsigned char smem_raw[];
+	T* smem = reinterpret_cast<T*>(smem_raw);
+	constexpr int EU = Unroll<MC>::EU;
 	Lane L;
-	if (!wave_item(g, L)) return;
+	if (!wave_item<NWV>(g, dst_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowq = (int64_t)g.H * g.W, rowv = (int64_t)g.H * g.Wv;
 	const T* qb = q + (int64_t)b * g.Tn * rowq;
@@ -237,65 +350,94 @@ __global__ __launch_bounds__(256) void sparse_bwd_dst(const T* __restrict__ dvo,
 
 	T qv[MC][VEC], dvod[MC][VEC], vbd[MC][VEC], X[MC][VEC], Y[MC][VEC], dvba[MC][VEC];
 	bool okq[MC], okv[MC];
+	int offq[MC], offv[MC];
 #pragma unroll
 	for (int m = 0; m < MC; m++) {
 		const int w0 = (m * G + L.sub) * VEC;
 		okq[m] = L.head_ok && w0 < g.W;
 		okv[m] = L.head_ok && w0 < g.Wv;
+		offq[m] = L.h * g.W + w0;
+		offv[m] = L.h * g.Wv + w0;
 #pragma unroll
 		for (int i = 0; i < VEC; i++) { qv[m][i] = 0; dvod[m][i] = 0; vbd[m][i] = 0; X[m][i] = 0; Y[m][i] = 0; dvba[m][i] = 0; }
-		if (okq[m]) ldv<T, VEC>(qb + (int64_t)L.tok * rowq + L.h * g.W + w0, qv[m]);
-		if (okv[m]) ldv<T, VEC>(dvob + (int64_t)L.tok * rowv + L.h * g.Wv + w0, dvod[m]);
-		if (BIDI && okv[m]) ldv<T, VEC>(vbk + ((int64_t)b * g.Tn + L.tok) * rowv + L.h * g.Wv + w0, vbd[m]);
+		if (okq[m]) ldv<T, VEC>(qb + (int64_t)L.tok * rowq + offq[m], qv[m]);
+		if (okv[m]) ldv<T, VEC>(dvob + (int64_t)L.tok * rowv + offv[m], dvod[m]);
+		if (BIDI && okv[m]) ldv<T, VEC>(vbk + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m], vbd[m]);
 	}
-	const int p0 = dst_ptr[L.tok], p1 = dst_ptr[L.tok + 1];
 	T S = 0;
-	for (int p = p0; p < p1; p++) {
-		const int src = csr_src[p];
-		T dp = 0;
-		T sg[MC][VEC], dvos[MC][VEC];
+	int sidx[EU];
 #pragma unroll
-		for (int m = 0; m < MC; m++) {
-			const int w0 = (m * G + L.sub) * VEC;
-			T kv[VEC], vs[VEC];
+	for (int u = 0; u < EU; u++) sidx[u] = L.pb < L.pe ? csr_src[min(L.pb + u, L.pe - 1)] : 0;
+	for (int p = L.pb; p < L.pe; p += EU) {
+		T kv[EU][MC][VEC], vs[EU][MC][VEC], dvos[EU][MC][VEC], pe[EU];
 #pragma unroll
-			for (int i = 0; i < VEC; i++) { kv[i] = qv[m][i]; vs[i] = 0; dvos[m][i] = 0; }
-			if (okq[m]) ldv<T, VEC>(kb + (int64_t)src * rowq + L.h * g.W + w0, kv);
-			if (okv[m]) ldv<T, VEC>(vb_ + (int64_t)src * rowv + L.h * g.Wv + w0, vs);
-			if (BIDI && okv[m]) ldv<T, VEC>(dvob + (int64_t)src * rowv + L.h * g.Wv + w0, dvos[m]);
+		for (int u = 0; u < EU; u++) {
+			pe[u] = L.head_ok ? Pb[(int64_t)min(p + u, L.pe - 1) * g.H + L.h] : (T)0;
 #pragma unroll
-			for (int i = 0; i < VEC; i++) {
-				dp += vs[i] * dvod[m][i];
-				if (BIDI) dp += vbd[m][i] * dvos[m][i];
-				sg[m][i] = sgn_t(qv[m][i] - kv[i]);
+			for (int m = 0; m < MC; m++) {
+#pragma unroll
+				for (int i = 0; i < VEC; i++) { kv[u][m][i] = qv[m][i]; vs[u][m][i] = 0; dvos[u][m][i] = 0; }
+				if (okq[m]) ldv<T, VEC>(kb + (int64_t)sidx[u] * rowq + offq[m], kv[u][m]);
+				if (okv[m]) ldv<T, VEC>(vb_ + (int64_t)sidx[u] * rowv + offv[m], vs[u][m]);
+				if (BIDI && okv[m]) ldv<T, VEC>(dvob + (int64_t)sidx[u] * rowv + offv[m], dvos[u][m]);
 			}
 		}
-		dp = group_sum(dp, G);
-		const T pe = L.head_ok ? Pb[(int64_t)p * g.H + L.h] : (T)0;
-		const T pd = pe * dp;
-		S += pd;
 #pragma unroll
-		for (int m = 0; m < MC; m++)
+		for (int u = 0; u < EU; u++) sidx[u] = csr_src[min(p + EU + u, L.pe - 1)];
+		T dp[EU];
 #pragma unroll
-			for (int i = 0; i < VEC; i++) {
-				X[m][i] += sg[m][i] * pd;
-				Y[m][i] += sg[m][i] * pe;
-				if (BIDI) dvba[m][i] += pe * dvos[m][i];
+		for (int u = 0; u < EU; u++) {
+			dp[u] = 0;
+#pragma unroll
+			for (int m = 0; m < MC; m++)
+#pragma unroll
+				for (int i = 0; i < VEC; i++) {
+					dp[u] += vs[u][m][i] * dvod[m][i];
+					if (BIDI) dp[u] += vbd[m][i] * dvos[u][m][i];
+				}
+		}
+#pragma unroll
+		for (int u = 0; u < EU; u++) dp[u] = group_sum(dp[u], G);
+#pragma unroll
+		for (int u = 0; u < EU; u++) {
+			if (p + u < L.pe) {  // uniform
+				const T pd = pe[u] * dp[u];
+				S += pd;
+#pragma unroll
+				for (int m = 0; m < MC; m++)
+#pragma unroll
+					for (int i = 0; i < VEC; i++) {
+						const T sg = sgn_t(qv[m][i] - kv[u][m][i]);
+						X[m][i] += sg * pd;
+						Y[m][i] += sg * pe[u];
+						if (BIDI) dvba[m][i] += pe[u] * dvos[u][m][i];
+					}
+				if (L.sub == 0 && L.head_ok) DAb[(int64_t)(p + u) * g.H + L.h] = dp[u];
 			}
-		if (L.sub == 0 && L.head_ok) DAb[(int64_t)p * g.H + L.h] = dp;
+		}
 	}
+	S = wg_sum<T, NWV>(S, smem, L.wave);
 #pragma unroll
-	for (int m = 0; m < MC; m++) {
-		const int w0 = (m * G + L.sub) * VEC;
-		T o[VEC];
+	for (int m = 0; m < MC; m++)
 #pragma unroll
-		for (int i = 0; i < VEC; i++) o[i] = use_softmax ? scale * (X[m][i] - S * Y[m][i]) : scale * X[m][i];
-		if (okq[m]) stv<T, VEC>(dq + ((int64_t)b * g.Tn + L.tok) * rowq + L.h * g.W + w0, o);
-		if (BIDI && okv[m]) stv<T, VEC>(dvb + ((int64_t)b * g.Tn + L.tok) * rowv + L.h * g.Wv + w0, dvba[m]);
+		for (int i = 0; i < VEC; i++) {
+			X[m][i] = wg_sum<T, NWV>(X[m][i], smem, L.wave);
+			if (use_softmax) Y[m][i] = wg_sum<T, NWV>(Y[m][i], smem, L.wave);
+			if (BIDI) dvba[m][i] = wg_sum<T, NWV>(dvba[m][i], smem, L.wave);
+		}
+	if (L.wave == 0 || NWV == 1) {
+#pragma unroll
+		for (int m = 0; m < MC; m++) {
+			T o[VEC];
+#pragma unroll
+			for (int i = 0; i < VEC; i++) o[i] = use_softmax ? scale * (X[m][i] - S * Y[m][i]) : scale * X[m][i];
+			if (okq[m]) stv<T, VEC>(dq + ((int64_t)b * g.Tn + L.tok) * rowq + offq[m], o);
+			if (BIDI && okv[m]) stv<T, VEC>(dvb + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m], dvba[m]);
+		}
 	}
 	__threadfence();  // dp values were stored by lane 0 of each head group
 	if (L.head_ok) {
-		for (int p = p0 + L.sub; p < p1; p += G) {
+		for (int p = L.pb + L.sub; p < L.pe; p += G) {
 			const int64_t ix = (int64_t)p * g.H + L.h;
 			const T pe = Pb[ix], dp = DAb[ix];
 			DAb[ix] = use_softmax ? pe * (dp - S) : pe * dp;
@@ -304,16 +446,18 @@ __global__ __launch_bounds__(256) void sparse_bwd_dst(const T* __restrict__ dvo,
 }
 
 // src pass: dv[src] = sum p * dvo[dst];  dk[src] = -scale * sum sign(q[dst]-k[src]) * da
-template <typename T, int VEC, int MC>
-__global__ __launch_bounds__(256) void sparse_bwd_src(const T* __restrict__ dvo, const T* __restrict__ q,
-                                                        const T* __restrict__ k, const int* __restrict__ src_ptr,
-                                                        const int* __restrict__ csc_dst,
-                                                        const int* __restrict__ csc_slot, const T* __restrict__ P,
-                                                        const T* __restrict__ DA, T* __restrict__ dv,
-                                                        T* __restrict__ dk, Geo g, T scale)
+template <typename T, int VEC, int MC, int NWV>
+__global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_src(
+    const T* __restrict__ dvo, const T* __restrict__ q, const T* __restrict__ k, const int* __restrict__ src_ptr,
+    const int* __restrict__ csc_dst, const int* __restrict__ csc_slot, const int* __restrict__ long_list,
+    const int* __restrict__ n_long, const T* __restrict__ P, const T* __restrict__ DA, T* __restrict__ dv,
+    T* __restrict__ dk, Geo g, T scale)
 {
+	extern __shared__ unsigned char smem_raw[];
+	T* smem = reinterpret_cast<T*>(smem_raw);
+	constexpr int EU = Unroll<MC>::EU;
 	Lane L;
-	if (!wave_item(g, L)) return;
+	if (!wave_item<NWV>(g, src_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowq = (int64_t)g.H * g.W, rowv = (int64_t)g.H * g.Wv;
 	const T* qb = q + (int64_t)b * g.Tn * rowq;
@@ -322,47 +466,78 @@ __global__ __launch_bounds__(256) void sparse_bwd_src(const T* __restrict__ dvo,
 	const T* DAb = DA + (int64_t)b * g.E * g.H;
 	T kv[MC][VEC], dva[MC][VEC], dka[MC][VEC];
 	bool okq[MC], okv[MC];
+	int offq[MC], offv[MC];
 #pragma unroll
 	for (int m = 0; m < MC; m++) {
 		const int w0 = (m * G + L.sub) * VEC;
 		okq[m] = L.head_ok && w0 < g.W;
 		okv[m] = L.head_ok && w0 < g.Wv;
+		offq[m] = L.h * g.W + w0;
+		offv[m] = L.h * g.Wv + w0;
 #pragma unroll
 		for (int i = 0; i < VEC; i++) { kv[m][i] = 0; dva[m][i] = 0; dka[m][i] = 0; }
-		if (okq[m]) ldv<T, VEC>(k + ((int64_t)b * g.Tn + L.tok) * rowq + L.h * g.W + w0, kv[m]);
+		if (okq[m]) ldv<T, VEC>(k + ((int64_t)b * g.Tn + L.tok) * rowq + offq[m], kv[m]);
 	}
-	const int i0 = src_ptr[L.tok], i1 = src_ptr[L.tok + 1];
-	for (int e = i0; e < i1; e++) {
-		const int dst = csc_dst[e], slot = csc_slot[e];
-		const int64_t ix = (int64_t)slot * g.H + L.h;
-		const T pe = L.head_ok ? Pb[ix] : (T)0;
-		const T da = L.head_ok ? DAb[ix] : (T)0;
+	int didx[EU], slot[EU];
 #pragma unroll
-		for (int m = 0; m < MC; m++) {
-			const int w0 = (m * G + L.sub) * VEC;
-			T qd[VEC], dd[VEC];
+	for (int u = 0; u < EU; u++) {
+		const int e = min(L.pb + u, L.pe - 1);
+		didx[u] = L.pb < L.pe ? csc_dst[e] : 0;
+		slot[u] = L.pb < L.pe ? csc_slot[e] : 0;
+	}
+	for (int e0 = L.pb; e0 < L.pe; e0 += EU) {
+		T qd[EU][MC][VEC], dd[EU][MC][VEC], pe[EU], da[EU];
 #pragma unroll
-			for (int i = 0; i < VEC; i++) { qd[i] = kv[m][i]; dd[i] = 0; }
-			if (okq[m]) ldv<T, VEC>(qb + (int64_t)dst * rowq + L.h * g.W + w0, qd);
-			if (okv[m]) ldv<T, VEC>(dvob + (int64_t)dst * rowv + L.h * g.Wv + w0, dd);
+		for (int u = 0; u < EU; u++) {
+			const int64_t ix = (int64_t)slot[u] * g.H + L.h;
+			pe[u] = L.head_ok ? Pb[ix] : (T)0;
+			da[u] = L.head_ok ? DAb[ix] : (T)0;
 #pragma unroll
-			for (int i = 0; i < VEC; i++) {
-				dva[m][i] += pe * dd[i];
-				dka[m][i] += sgn_t(qd[i] - kv[m][i]) * da;
+			for (int m = 0; m < MC; m++) {
+#pragma unroll
+				for (int i = 0; i < VEC; i++) { qd[u][m][i] = kv[m][i]; dd[u][m][i] = 0; }
+				if (okq[m]) ldv<T, VEC>(qb + (int64_t)didx[u] * rowq + offq[m], qd[u][m]);
+				if (okv[m]) ldv<T, VEC>(dvob + (int64_t)didx[u] * rowv + offv[m], dd[u][m]);
 			}
 		}
+#pragma unroll
+		for (int u = 0; u < EU; u++) {
+			const int e = min(e0 + EU + u, L.pe - 1);
+			didx[u] = csc_dst[e];
+			slot[u] = csc_slot[e];
+		}
+#pragma unroll
+		for (int u = 0; u < EU; u++)
+			if (e0 + u < L.pe)
+#pragma unroll
+				for (int m = 0; m < MC; m++)
+#pragma unroll
+					for (int i = 0; i < VEC; i++) {
+						dva[m][i] += pe[u] * dd[u][m][i];
+						dka[m][i] += sgn_t(qd[u][m][i] - kv[m][i]) * da[u];
+					}
 	}
 #pragma unroll
-	for (int m = 0; m < MC; m++) {
-		const int w0 = (m * G + L.sub) * VEC;
+	for (int m = 0; m < MC; m++)
 #pragma unroll
-		for (int i = 0; i < VEC; i++) dka[m][i] *= -scale;
-		if (okv[m]) stv<T, VEC>(dv + ((int64_t)b * g.Tn + L.tok) * rowv + L.h * g.Wv + w0, dva[m]);
-		if (okq[m]) stv<T, VEC>(dk + ((int64_t)b * g.Tn + L.tok) * rowq + L.h * g.W + w0, dka[m]);
+		for (int i = 0; i < VEC; i++) {
+			dva[m][i] = wg_sum<T, NWV>(dva[m][i], smem, L.wave);
+			dka[m][i] = wg_sum<T, NWV>(dka[m][i], smem, L.wave);
+		}
+	if (L.wave == 0 || NWV == 1) {
+#pragma unroll
+		for (int m = 0; m < MC; m++) {
+#pragma unroll
+			for (int i = 0; i < VEC; i++) dka[m][i] *= -scale;
+			if (okv[m]) stv<T, VEC>(dv + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m], dva[m]);
+			if (okq[m]) stv<T, VEC>(dk + ((int64_t)b * g.Tn + L.tok) * rowq + offq[m], dka[m]);
+		}
 	}
 }
 
 // ---------------------------------------------------------------------------------- host side
+
+constexpr int LONG_NWV = 8;  // waves that share one long segment
 
 struct Shape {
 	int64_t B, T, H, W, Wv, E;
@@ -371,17 +546,19 @@ struct Shape {
 struct Cfg {
 	int vec, mc;
 	Geo g;
-	dim3 grid, block;
+	dim3 grid, block;            // wave-per-item launch
+	dim3 lgrid, lblock;          // workgroup-per-long-segment launch (only when g.long_on)
+	const int *long_dst, *long_src, *n_long_dst, *n_long_src;
+	const int *dst_ptr, *src_ptr, *csr_src, *csc_dst, *csc_slot;
 };
 
-int make_cfg(const Shape& s, size_t elt, const void* const* ptrs, int n_ptrs, Cfg& c)
+int make_cfg(const Shape& s, const void* plan, const void* const* ptrs, int n_ptrs, Cfg& c)
 {
 	if (s.B < 0 || s.T < 0 || s.H < 0 || s.W < 1 || s.Wv < 1 || s.E < 0) return L1ATTN_ERR_ARG;
 	if (s.T > (1LL << 30) || s.E > 2147483647LL - 4096 || s.B > 65535 || s.H > 32768) return L1ATTN_ERR_RANGE;
 	bool aligned = true;
 	for (int i = 0; i < n_ptrs; i++) aligned = aligned && ((((uintptr_t)ptrs[i]) & 15) == 0);
 	c.vec = (s.W % 4 == 0 && s.Wv % 4 == 0 && aligned) ? 4 : 1;
-	(void)elt;
 	const int64_t wmax = s.W > s.Wv ? s.W : s.Wv;
 	int64_t chunks = l1_cdiv(wmax, c.vec);
 	if (chunks > 256) return L1ATTN_ERR_RANGE;
@@ -393,18 +570,39 @@ int make_cfg(const Shape& s, size_t elt, const void* const* ptrs, int n_ptrs, Cf
 	c.g.log2G = lg;
 	c.g.n_hc = (int)l1_cdiv(s.H, 64 >> lg);
 	const int64_t items = s.T * c.g.n_hc;
-	if (l1_cdiv(items, 4) > 2147483647LL) return L1ATTN_ERR_RANGE;
+	if (l1_cdiv(items, 4) > 2147483647LL || c.g.n_hc > 65535) return L1ATTN_ERR_RANGE;
 	c.grid = dim3((unsigned)l1_cdiv(items, 4), (unsigned)s.B, 1);
 	c.block = dim3(256);
+	const PlanLayout L = plan_layout(s.E, s.T);
+	const int* words = (const int*)plan;
+	// a list of E edges has at most E / PLAN_LONG_SEGMENT long segments: that bounds the second launch
+	c.g.long_on = (c.mc == 1 && s.E > PLAN_LONG_SEGMENT) ? 1 : 0;
+	c.lgrid = dim3((unsigned)L.long_cap, (unsigned)s.B, (unsigned)c.g.n_hc);
+	c.lblock = dim3(64 * LONG_NWV);
+	c.long_dst = words + L.long_dst;
+	c.long_src = words + L.long_src;
+	c.n_long_dst = words + PLAN_H_NLONG_DST;
+	c.n_long_src = words + PLAN_H_NLONG_SRC;
+	c.dst_ptr = words + L.dst_ptr;
+	c.src_ptr = words + L.src_ptr;
+	c.csr_src = words + L.csr_src;
+	c.csc_dst = words + L.csc_dst;
+	c.csc_slot = words + L.csc_slot;
 	return L1ATTN_OK;
 }
 
-#define DISPATCH_VM(cfg, CALL)                      \
-	do {                                            \
-		if ((cfg).vec == 4 && (cfg).mc == 1) { CALL(4, 1); } \
-		else if ((cfg).vec == 4) { CALL(4, 4); }    \
-		else if ((cfg).mc == 1) { CALL(1, 1); }     \
-		else { CALL(1, 4); }                        \
+// CALL(VEC, MC, NWV, grid, block, lds_bytes)
+#define DISPATCH_VM(cfg, T, CALL)                                                          \
+	do {                                                                                   \
+		if ((cfg).vec == 4 && (cfg).mc == 1) { CALL(4, 1, 1, (cfg).grid, (cfg).block, 0); } \
+		else if ((cfg).vec == 4) { CALL(4, 4, 1, (cfg).grid, (cfg).block, 0); }            \
+		else if ((cfg).mc == 1) { CALL(1, 1, 1, (cfg).grid, (cfg).block, 0); }             \
+		else { CALL(1, 4, 1, (cfg).grid, (cfg).block, 0); }                                \
+		if ((cfg).g.long_on) {                                                             \
+			const size_t lds__ = (size_t)LONG_NWV * 64 * sizeof(T);                        \
+			if ((cfg).vec == 4) { CALL(4, 1, LONG_NWV, (cfg).lgrid, (cfg).lblock, lds__); } \
+			else { CALL(1, 1, LONG_NWV, (cfg).lgrid, (cfg).lblock, lds__); }               \
+		}                                                                                  \
 	} while (0)
 
 template <typename T>
@@ -415,22 +613,20 @@ int sparse_fwd_impl(const T* v, const T* vbk, const T* q, const T* k, const void
 	if (!v || !q || !k || !plan || !vo || (s.E > 0 && !P) || (bidi && !vbk)) return L1ATTN_ERR_ARG;
 	const void* ptrs[] = {v, vbk, q, k, vo};
 	Cfg c;
-	int rc = make_cfg(s, sizeof(T), ptrs, 5, c);
+	int rc = make_cfg(s, plan, ptrs, 5, c);
 	if (rc) return rc;
-	const PlanLayout L = plan_layout(s.E, s.T);
-	const int* words = (const int*)plan;
 	const T scale = (T)(-1.0 / sqrt((double)s.W));
-#define CALL(V, M)                                                                                               \
-	hipLaunchKernelGGL((sparse_fwd_dst<T, V, M>), c.grid, c.block, 0, st, v, q, k, words + L.dst_ptr,            \
-	                   words + L.csr_src, vo, P, c.g, use_softmax, scale)
-	DISPATCH_VM(c, CALL);
+#define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
+	hipLaunchKernelGGL((sparse_fwd_dst<T, V, M, N>), GRID, BLOCK, LDS, st, v, q, k, c.dst_ptr, c.csr_src,        \
+	                   c.long_dst, c.n_long_dst, vo, P, c.g, use_softmax, scale)
+	DISPATCH_VM(c, T, CALL);
 #undef CALL
 	L1_LAUNCH_CHECK();
 	if (bidi) {
-#define CALL(V, M)                                                                                               \
-	hipLaunchKernelGGL((sparse_fwd_src<T, V, M>), c.grid, c.block, 0, st, vbk, words + L.src_ptr,                \
-	                   words + L.csc_dst, words + L.csc_slot, (const T*)P, vo, c.g)
-		DISPATCH_VM(c, CALL);
+#define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
+	hipLaunchKernelGGL((sparse_fwd_src<T, V, M, N>), GRID, BLOCK, LDS, st, vbk, c.src_ptr, c.csc_dst,            \
+	                   c.csc_slot, c.long_src, c.n_long_src, (const T*)P, vo, c.g)
+		DISPATCH_VM(c, T, CALL);
 #undef CALL
 		L1_LAUNCH_CHECK();
 	}
@@ -446,29 +642,27 @@ int sparse_bwd_impl(const T* dvo, const T* v, const T* vbk, const T* q, const T*
 		return L1ATTN_ERR_ARG;
 	const void* ptrs[] = {dvo, v, vbk, q, k, dv, dvb, dq, dk};
 	Cfg c;
-	int rc = make_cfg(s, sizeof(T), ptrs, 9, c);
+	int rc = make_cfg(s, plan, ptrs, 9, c);
 	if (rc) return rc;
-	const PlanLayout L = plan_layout(s.E, s.T);
-	const int* words = (const int*)plan;
 	const T scale = (T)(-1.0 / sqrt((double)s.W));
 	if (bidi) {
-#define CALL(V, M)                                                                                               \
-	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, true>), c.grid, c.block, 0, st, dvo, v, vbk, q, k,               \
-	                   words + L.dst_ptr, words + L.csr_src, P, DA, dq, dvb, c.g, use_softmax, scale)
-		DISPATCH_VM(c, CALL);
+#define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
+	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, true, N>), GRID, BLOCK, LDS, st, dvo, v, vbk, q, k, c.dst_ptr,   \
+	                   c.csr_src, c.long_dst, c.n_long_dst, P, DA, dq, dvb, c.g, use_softmax, scale)
+		DISPATCH_VM(c, T, CALL);
 #undef CALL
 	} else {
-#define CALL(V, M)                                                                                               \
-	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, false>), c.grid, c.block, 0, st, dvo, v, vbk, q, k,              \
-	                   words + L.dst_ptr, words + L.csr_src, P, DA, dq, dvb, c.g, use_softmax, scale)
-		DISPATCH_VM(c, CALL);
+#define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
+	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, false, N>), GRID, BLOCK, LDS, st, dvo, v, vbk, q, k, c.dst_ptr,  \
+	                   c.csr_src, c.long_dst, c.n_long_dst, P, DA, dq, dvb, c.g, use_softmax, scale)
+		DISPATCH_VM(c, T, CALL);
 #undef CALL
 	}
 	L1_LAUNCH_CHECK();
-#define CALL(V, M)                                                                                               \
-	hipLaunchKernelGGL((sparse_bwd_src<T, V, M>), c.grid, c.block, 0, st, dvo, q, k, words + L.src_ptr,          \
-	                   words + L.csc_dst, words + L.csc_slot, P, (const T*)DA, dv, dk, c.g, scale)
-	DISPATCH_VM(c, CALL);
+#define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
+	hipLaunchKernelGGL((sparse_bwd_src<T, V, M, N>), GRID, BLOCK, LDS, st, dvo, q, k, c.src_ptr, c.csc_dst,      \
+	                   c.csc_slot, c.long_src, c.n_long_src, P, (const T*)DA, dv, dk, c.g, scale)
+	DISPATCH_VM(c, T, CALL);
 #undef CALL
 	L1_LAUNCH_CHECK();
 	return L1ATTN_OK;

@@ -234,6 +234,36 @@ def test_sparse_permutation_invariance_and_determinism():
     assert torch.equal(ru[0], rb[0]) and torch.equal(ru[1], rb[1])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_sparse_long_segments_vs_oracle(dtype):
+    """Segments longer than 128 edges are walked by a whole workgroup (eight waves, fixed-order
+    combine): a hub dst with 700 incoming edges, a hub src with 500 outgoing ones, duplicates, and a
+    segment of exactly 128 and 129 edges on either side of the threshold."""
+    print("case sparse long segments", dtype, flush=True)
+    g = torch.Generator().manual_seed(77)
+    B, T, H, W = 2, 300, 4, 16
+    rows = [torch.stack((torch.full((700,), 5), torch.randint(0, T, (700,), generator=g)), 1),
+            torch.stack((torch.randint(0, T, (500,), generator=g), torch.full((500,), 9)), 1),
+            torch.stack((torch.full((128,), 20), torch.arange(128)), 1),
+            torch.stack((torch.full((129,), 21), torch.arange(129)), 1),
+            torch.randint(0, T, (400, 2), generator=g)]
+    co = torch.cat(rows, 0)
+    co = co[torch.randperm(co.shape[0], generator=g)]
+    coo, dmx, smx = oracle.expand_coo(co)
+    assert dmx > 700 and smx > 500
+    v, vb, q, k, dvo = (torch.randn(B, T, H, W, generator=g, dtype=dtype) for _ in range(5))
+    f32 = dtype == torch.float32
+    for sm in (True, False):
+        _check(_run_uni(v, q, k, coo, dmx, sm, dvo), _oracle_uni(v, q, k, coo, dmx, sm, dvo, 1),
+               [FWD_TOL] + [BWD_TOL] * 3 if f32 else [F64_TOL] * 4)
+        _check(_run_bidi(v, vb, q, k, coo, dmx, sm, dvo), _oracle_bidi(v, vb, q, k, coo, dmx, sm, dvo, 1),
+               [FWD_TOL] + [BWD_TOL] * 4 if f32 else [F64_TOL] * 5)
+    r1 = _run_bidi(v, vb, q, k, coo, dmx, True, dvo)
+    r2 = _run_bidi(v, vb, q, k, coo, dmx, True, dvo)
+    for a, b in zip(r1, r2):
+        assert torch.equal(a, b)
+
+
 def test_sparse_value_width_differs_from_key_width():
     # allowed by the reference's CUDA path (v_width, cuda/l1attn_sparse_cuda_kernel.cu:385)
     print("case sparse Wv != W", flush=True)
