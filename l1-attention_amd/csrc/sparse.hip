@@ -66,6 +66,15 @@ template <> __device__ __forceinline__ double exp_t<double>(double x) { return e
 template <typename T> __device__ __forceinline__ T abs_t(T x) { return x < (T)0 ? -x : x; }
 template <typename T> __device__ __forceinline__ T sgn_t(T x) { return (T)((x > (T)0) - (x < (T)0)); }
 
+// Orders a wave's own global stores before its later loads of the same addresses from other lanes.
+// Workgroup scope is enough (the data never leaves the wave) and, unlike an agent-scope fence, does
+// not write back the L2.
+__device__ __forceinline__ void wave_store_load_fence()
+{
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
 // geometry of one work item, shared by all kernels
 struct Geo {
 	int Tn, H, W, Wv, E;
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_dst(
 		}
 	}
 	// the weights below were stored by lane 0 of each head group: make them visible to its other lanes
-	__threadfence();
+	wave_store_load_fence();
 	if (use_softmax && L.head_ok) {
 		// normalise the stored weights of this wave's share; the G lanes of a head take every G-th slot
 		for (int p = L.pb + L.sub; p < L.pe; p += G) Pb[(int64_t)p * g.H + L.h] *= inv;
@@ -435,7 +444,7 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_dst(
 			if (BIDI && okv[m]) stv<T, VEC>(dvb + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m], dvba[m]);
 		}
 	}
-	__threadfence();  // dp values were stored by lane 0 of each head group
+	wave_store_load_fence();  // dp values were stored by lane 0 of each head group
 	if (L.head_ok) {
 		for (int p = L.pb + L.sub; p < L.pe; p += G) {
 			const int64_t ix = (int64_t)p * g.H + L.h;
