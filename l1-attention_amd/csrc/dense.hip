@@ -93,6 +93,7 @@ __global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict_
 // ------------------------------------------------------------------------------------------
 
 constexpr int FWD_SJ = 8;  // src rows finished between two output flushes
+constexpr int FWD_TILE = 1024 + 4 * WAVE;  // floats per staged src row: 64*NW outputs + one pad column per sub-tile (NH >= 4)
 
 // Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.
 // This maps the flat dispatch index to a logical one such that logically consecutive workgroups
@@ -112,22 +113,26 @@ __device__ __forceinline__ LogicalBlock xcd_remap()
 	return lb;
 }
 
-// grid.x = dst tiles of 64 tokens, grid.y = src chunks, grid.z = B * head groups.
-// block = 64 * NW threads, NW = heads per group (<= 16); wave w of the block owns head hg*NW + w.
+// grid.x = dst tiles of 64*NTS tokens, grid.y = src chunks, grid.z = B * head groups.
+// block = 64 * NW threads (NW <= 16 waves) = NH heads x NTS dst sub-tiles of 64 tokens: wave w owns head
+// hg*NH + w % NH and sub-tile w / NH.  Waves of the same head stream the same k rows, so the second one
+// finds them in the scalar cache.
 // W is a compile-time multiple of 16; q and k must be 16-byte aligned.
 template <int W>
 __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restrict__ q, const float* __restrict__ k,
                                                              float* __restrict__ attn, int Tn, int H, int n_hg,
-                                                             int s_chunk, float scale)
+                                                             int NH, int s_chunk, float scale)
 {
-	__shared__ float tile[FWD_SJ][WAVE * 17];
+	__shared__ float tile[FWD_SJ][FWD_TILE];
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const int NW = blockDim.x >> 6;
+	const int NW = blockDim.x >> 6, NTS = NW / NH, PH = NH + 1;
 	const LogicalBlock lb = xcd_remap();
 	const int b = lb.z / n_hg, hg = lb.z % n_hg;
-	const int h = min(hg * NW + wave, H - 1);  // surplus waves of the last group redo head H-1, never stored
-	const int t0 = lb.x * WAVE;
+	const int hl = wave % NH, ts = wave / NH;
+	const int h = min(hg * NH + hl, H - 1);  // surplus waves of the last group redo head H-1, never stored
+	const int tg0 = lb.x * NTS * WAVE;       // first dst token of the workgroup
+	const int t0 = tg0 + ts * WAVE;          // first dst token of this wave
 	const int t = min(t0 + lane, Tn - 1);
 
 	float qr[W];
@@ -140,10 +145,10 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 		}
 	}
 
-	// output role of this thread in the flush: element e = threadIdx.x of the [64 x NW] row tile
-	const int o_tl = threadIdx.x / NW, o_hh = threadIdx.x % NW;
-	const bool o_ok = (t0 + o_tl < Tn) && (hg * NW + o_hh < H);
-	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (t0 + o_tl)) * H + hg * NW + o_hh;
+	// output role of this thread in the flush: element e = threadIdx.x of the [64*NTS x NH] row tile
+	const int o_tl = threadIdx.x / NH, o_hh = threadIdx.x % NH;
+	const bool o_ok = (tg0 + o_tl < Tn) && (hg * NH + o_hh < H);
+	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (tg0 + o_tl)) * H + hg * NH + o_hh;
 	const int64_t o_pitch = (int64_t)Tn * H;
 
 	const int s_begin = lb.y * s_chunk;
@@ -156,13 +161,13 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 			float a = 0.0f;
 #pragma unroll
 			for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
-			tile[j][lane * 17 + wave] = a * scale;
+			tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
 		}
 		__syncthreads();
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
 			const int s = s0 + j;
-			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * 17 + o_hh];
+			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * PH + o_hh];
 		}
 		__syncthreads();
 	}
@@ -189,17 +194,19 @@ __device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
 template <int W>
 __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restrict__ q, const float* __restrict__ k,
                                                              float* __restrict__ attn, int Tn, int H, int n_hg,
-                                                             int s_chunk, float scale)
+                                                             int NH, int s_chunk, float scale)
 {
 	static_assert(W % 32 == 0 && (FWD_SJ % 2) == 0, "chunk stream must keep buffer parity across src blocks");
-	__shared__ float tile[FWD_SJ][WAVE * 17];
+	__shared__ float tile[FWD_SJ][FWD_TILE];
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const int NW = blockDim.x >> 6;
+	const int NW = blockDim.x >> 6, NTS = NW / NH, PH = NH + 1;
 	const LogicalBlock lb = xcd_remap();
 	const int b = lb.z / n_hg, hg = lb.z % n_hg;
-	const int h = min(hg * NW + wave, H - 1);
-	const int t0 = lb.x * WAVE;
+	const int hl = wave % NH, ts = wave / NH;
+	const int h = min(hg * NH + hl, H - 1);  // surplus waves of the last group redo head H-1, never stored
+	const int tg0 = lb.x * NTS * WAVE;       // first dst token of the workgroup
+	const int t0 = tg0 + ts * WAVE;          // first dst token of this wave
 	const int t = min(t0 + lane, Tn - 1);
 
 	float qr[W];
@@ -211,9 +218,9 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
 		}
 	}
-	const int o_tl = threadIdx.x / NW, o_hh = threadIdx.x % NW;
-	const bool o_ok = (t0 + o_tl < Tn) && (hg * NW + o_hh < H);
-	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (t0 + o_tl)) * H + hg * NW + o_hh;
+	const int o_tl = threadIdx.x / NH, o_hh = threadIdx.x % NH;
+	const bool o_ok = (tg0 + o_tl < Tn) && (hg * NH + o_hh < H);
+	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (tg0 + o_tl)) * H + hg * NH + o_hh;
 	const int64_t o_pitch = (int64_t)Tn * H;
 
 	constexpr int CPR = W / 32;          // chunks per k row
@@ -258,13 +265,13 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 #pragma unroll
 				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b1h[i]);
 			}
-			if (part == CPR - 1) tile[j][lane * 17 + wave] = a * scale;
+			if (part == CPR - 1) tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
 		}
 		__syncthreads();
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
 			const int s = s0 + j;
-			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * 17 + o_hh];
+			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * PH + o_hh];
 		}
 		__syncthreads();
 	}
@@ -487,22 +494,35 @@ int launch_bwd_generic(const T* dA, const T* q, const T* k, T* dq, T* dk, int64_
 	return L1ATTN_OK;
 }
 
+// heads per workgroup and dst sub-tiles per workgroup of the fast forward.  All heads of a dst tile
+// in one workgroup keeps the output runs whole 64-byte lines; splitting the heads over two
+// workgroups (NH 8, NTS 2, two waves sharing each k row) measured slower.
+void fwd_shape(int64_t H, int64_t T, int& NH, int& NTS)
+{
+	(void)T;
+	NH = (int)(H < 16 ? H : 16);
+	NTS = 1;
+}
+
 // fast forward: W a multiple of 16 up to 128, 16-byte aligned rows, at least half a wave of tokens
 bool fwd_fast_ok(const float* q, const float* k, int64_t B, int64_t T, int64_t H, int64_t W)
 {
 	if (W < 16 || W > 128 || (W % 16) != 0 || T < 32) return false;
 	if ((((uintptr_t)q) | ((uintptr_t)k)) & 15) return false;
-	const int64_t NW = H < 16 ? H : 16;
-	const int64_t n_hg = l1_cdiv(H, NW);
+	int NH, NTS;
+	fwd_shape(H, T, NH, NTS);
+	const int64_t n_hg = l1_cdiv(H, NH);
 	return B * n_hg <= 65535 && T <= (1 << 30) && H <= 65535;
 }
 
 int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int64_t Tn, int64_t H, int64_t W,
                     hipStream_t st)
 {
-	const int NW = (int)(H < 16 ? H : 16);
-	const int n_hg = (int)l1_cdiv(H, NW);
-	const int n_tt = (int)l1_cdiv(Tn, WAVE);
+	int NH, NTS;
+	fwd_shape(H, Tn, NH, NTS);
+	const int NW = NH * NTS;
+	const int n_hg = (int)l1_cdiv(H, NH);
+	const int n_tt = (int)l1_cdiv(Tn, WAVE * NTS);
 	// split the src range so that the launch has a few thousand workgroups, in multiples of FWD_SJ
 	int64_t want_chunks = l1_cdiv(2048, (int64_t)n_tt * B * n_hg);
 	int64_t s_chunk = l1_cdiv(l1_cdiv(Tn, want_chunks), FWD_SJ) * FWD_SJ;
@@ -513,7 +533,7 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 	dim3 grid(n_tt, n_sc, (unsigned)(B * n_hg)), block(64 * NW);
 #define L1_FWD_CASE(KERNEL, WV)                                                                                  \
 	case WV:                                                                                                     \
-		hipLaunchKernelGGL(KERNEL<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, (int)s_chunk,        \
+		hipLaunchKernelGGL(KERNEL<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, NH, (int)s_chunk,    \
 		                   scale);                                                                               \
 		break
 	switch (W) {
