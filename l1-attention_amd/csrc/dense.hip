@@ -26,6 +26,14 @@ namespace {
 
 constexpr int WAVE = 64;
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global store (vmcnt(0)), which stalls the workgroup for a full HBM write round trip each time a
+// barrier follows stores; here only the LDS/scalar counter is drained before the barrier.
+__device__ __forceinline__ void lds_barrier()
+{
+	asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ------------------------------------------------------------------------------------------
 // generic kernels
 // ------------------------------------------------------------------------------------------
@@ -163,13 +171,13 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 			for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
 			tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
 		}
-		__syncthreads();
+		lds_barrier();
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
 			const int s = s0 + j;
-			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * PH + o_hh];
+			if (o_ok && s < s_end) __builtin_nontemporal_store(tile[j][o_tl * PH + o_hh], &o_base[s * o_pitch]);
 		}
-		__syncthreads();
+		lds_barrier();
 	}
 }
 
@@ -267,13 +275,13 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 			}
 			if (part == CPR - 1) tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
 		}
-		__syncthreads();
+		lds_barrier();
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
 			const int s = s0 + j;
-			if (o_ok && s < s_end) o_base[s * o_pitch] = tile[j][o_tl * PH + o_hh];
+			if (o_ok && s < s_end) __builtin_nontemporal_store(tile[j][o_tl * PH + o_hh], &o_base[s * o_pitch]);
 		}
-		__syncthreads();
+		lds_barrier();
 	}
 	swait32(b0l, b0h);  // drain the last prefetch before the wave ends
 }
@@ -391,7 +399,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	prefetch(0);
 
 	for (int s0 = 0; s0 < Tn; s0 += BWD_SJ) {
-		__syncthreads();  // the previous step's LDS reads are done
+		lds_barrier();  // the previous step's LDS reads are done
 #pragma unroll
 		for (int r = 0; r < PER; r++)
 			if (st_lds[r] >= 0) gl[st_lds[r]] = g_pre[r];
@@ -401,7 +409,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			kc[j] = k_pre[j] * BWD_PRESCALE;
 			dka[j] = 0.0f;
 		}
-		__syncthreads();
+		lds_barrier();
 		if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
 		{
 			// all dA values of this step for the lane's head, read one float4 ahead of their use
