@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per dense-backward launch (B=8,T=4096,H=16,W=64) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/dense_B8_T4096_H16_W64_pmc_*.txt), scaled by what three 1 GiB device copies read on the same
 # counters (profiles/copy_1GiB_pmc_*.txt: FETCH_SIZE 0.5 per KiB -> x2.0, WRITE_SIZE 1.0 per KiB -> x1.0):
-# main kernel 4925279*2 + 8519680 KiB, dk reduce 4194587*2 + 131072 KiB.
-DENSE_BWD_TRAFFIC_BYTES = (4925279 * 2 + 8519680 + 4194587 * 2 + 131072) * 1024
+# main kernel 5291015*2 + 8519680 KiB, dk reduce 4194591*2 + 131072 KiB.
+DENSE_BWD_TRAFFIC_BYTES = (5291015 * 2 + 8519680 + 4194591 * 2 + 131072) * 1024
 
 
 def log(*a):
