@@ -7,6 +7,7 @@ code (-packed-fp32-ops): the kernels issue scalar-per-lane fp32 VALU operations 
 """
 import glob
 import os
+import re
 import subprocess
 import sys
 
@@ -17,6 +18,62 @@ ARCH = "gfx950"
 
 def sources():
     return sorted(glob.glob(os.path.join(HERE, "csrc", "*.hip")))
+
+
+def _sregs(tok):
+    m = re.match(r"s\[(\d+):(\d+)\]$", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"s(\d+)$", tok)
+    return {int(m.group(1))} if m else set()
+
+
+def check_scalar_prefetch(asm_text, kernel_substr="dense_fwd_f32_pipe"):
+    """Static check of the generated ISA of the software-pipelined forward kernels.
+
+    Those kernels issue `s_load_dwordx16` from inline asm and wait for it one chunk of math later.
+    The compiler does not know that the destination SGPRs are written asynchronously: if register
+    pressure makes it spill, copy or reuse them between the load and the next `s_waitcnt lgkmcnt(0)`,
+    the late-arriving data lands in whatever lives there by then (a pointer, an exec mask) and the
+    kernel faults.  This walks every such kernel and fails the build if any instruction reads or
+    writes an SGPR that still has a scalar load in flight, or if the kernel ends with one in flight.
+    Returns the number of prefetch loads checked."""
+    cur, inflight, n_loads, problems = None, set(), 0, []
+    for ln, line in enumerate(asm_text.split("\n"), 1):
+        l = line.strip()
+        if l.startswith("_Z") and ":" in l.split(";")[0]:
+            cur, inflight = l.split(":")[0], set()
+            continue
+        if cur is None or kernel_substr not in cur or not l or l[0] in ";.":
+            continue
+        l = l.split(";")[0].strip()
+        if not l:
+            continue
+        op = l.split()[0]
+        toks = re.findall(r"s\[\d+:\d+\]|s\d+", l)
+        used = set()
+        for t in toks:
+            used |= _sregs(t)
+        if op.startswith("s_load_dword") or op.startswith("s_buffer_load"):
+            src = set()
+            for t in toks[1:]:
+                src |= _sregs(t)
+            if src & inflight:
+                problems.append((cur, ln, l))
+            inflight |= _sregs(toks[0]) if toks else set()
+            n_loads += 1
+        elif op == "s_waitcnt" and "lgkmcnt(0)" in l:
+            inflight = set()
+        elif op == "s_endpgm":
+            if inflight:
+                problems.append((cur, ln, "s_endpgm with scalar loads in flight"))
+            inflight = set()
+        elif used & inflight:
+            problems.append((cur, ln, l))
+    if problems:
+        msg = "\n".join("%s line %d: %s" % p for p in problems[:10])
+        raise RuntimeError("scalar-prefetch check failed: SGPRs touched while their s_load is in flight\n" + msg)
+    return n_loads
 
 
 def build(verbose=False):
@@ -41,6 +98,17 @@ def build(verbose=False):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if verbose and out.strip():
             print(out)
+    # ISA-level safety check of the kernels that prefetch through inline-asm scalar loads
+    dense = os.path.join(HERE, "csrc", "dense.hip")
+    asm = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-Xclang", "-target-feature",
+                          "-Xclang", "-packed-fp32-ops", "-I", os.path.join(HERE, "csrc"), "-S",
+                          "--cuda-device-only", dense, "-o", "-"],
+                         check=True, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True).stdout
+    n = check_scalar_prefetch(asm)
+    if n < 8:
+        raise RuntimeError("scalar-prefetch check found no pipelined forward kernel to verify")
+    if verbose:
+        print("scalar-prefetch check: %d loads verified" % n)
     cmd = [hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd))

@@ -91,3 +91,29 @@ def test_binding_rejects_cpu_tensors():
         drv.dense_forward(q, q)
     with pytest.raises(RuntimeError, match="d_attn must be a CUDA tensor"):
         drv.dense_backward(torch.randn(1, 4, 4, 2), q, q)
+
+
+def test_build_rejects_sgprs_touched_under_a_scalar_load_in_flight():
+    """build.py's ISA check of the software-pipelined forward kernels: an SGPR spill between an
+    inline-asm s_load and its wait must fail the build (such code faults on the GPU)."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import build
+    good = """
+_ZN1_18dense_fwd_f32_pipeILi64EEEv: ; @k
+	s_load_dwordx16 s[36:51], s[0:1], 0x0
+	v_subrev_f32_e32 v1, s4, v2
+	s_waitcnt lgkmcnt(0)
+	v_subrev_f32_e32 v1, s36, v2
+	s_endpgm
+"""
+    assert build.check_scalar_prefetch(good) == 1
+    for bad_line in ("v_writelane_b32 v88, s40, 3", "v_readlane_b32 s51, v90, 11", "s_mov_b32 s36, s2",
+                     "v_subrev_f32_e32 v1, s37, v2"):
+        bad = good.replace("	v_subrev_f32_e32 v1, s4, v2", "	" + bad_line)
+        with pytest.raises(RuntimeError, match="in flight"):
+            build.check_scalar_prefetch(bad)
+    with pytest.raises(RuntimeError, match="in flight"):
+        build.check_scalar_prefetch(good.replace("	s_waitcnt lgkmcnt(0)\n", ""))
+    # kernels without the prefetch idiom are not inspected
+    assert build.check_scalar_prefetch(good.replace("dense_fwd_f32_pipe", "other_kernel")) == 0
