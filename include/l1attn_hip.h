@@ -57,7 +57,11 @@ int l1attn_dense_fwd_f64(const double* q, const double* k, double* attn,
  * l1attn_dense_bwd_workspace_bytes() for full speed; any multiple of one batch's share works,
  * the batches are then processed in several launches).  The f64 entry needs no workspace.
  * f32 fast path: sign() is taken from (q-k)*2^64, exact for |q|,|k| < 2^63 and differences
- * that are 0 or at least 2^-64 in magnitude.
+ * that are 0 or at least 2^-64 in magnitude.  For 2048 <= T <= 8192 (and enough work to fill
+ * the GPU) sign() is taken from the column ranks of l1attn_dense_column_ranks_f32 instead, exact
+ * for all finite inputs; the gradient is then assembled as 2*sum(hv*d_attn) - sum(d_attn) with
+ * hv = (sign+1)/2, so an element whose pairs all tie comes out as a rounding residue of the two
+ * sums (about 1e-6 of the largest gradient) instead of an exact zero.
  */
 size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W);
 int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk,
@@ -66,6 +70,18 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k, double* dq, double* dk,
                          int64_t B, int64_t T, int64_t H, int64_t W,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Order-preserving integer ranks of q and k per column (b,h,w), the first stage of the f32
+ * backward for T <= 8192: rq[b,t,h,w] - (rk[b,s,h,w] + 1/2) has the sign of q[b,t,h,w] -
+ * k[b,s,h,w], is 0 exactly when they are equal (-0 == +0) and is at least 1 in magnitude
+ * otherwise; rk holds its rank minus one half.  rq, rk: [B,T,H,W] floats.
+ * No counterpart in the reference, which evaluates sign(q-k) per pair-element
+ * (cuda/l1attn_cuda_kernel.cu:206-455); exported so that the stage can be tested on its own.
+ * Returns L1ATTN_ERR_RANGE for T > 8192.
+ */
+int l1attn_dense_column_ranks_f32(const float* q, const float* k, float* rq, float* rk,
+                                  int64_t B, int64_t T, int64_t H, int64_t W, void* stream);
 
 /* -------------------------------------------------------------------------- edge lists */
 

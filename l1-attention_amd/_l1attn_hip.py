@@ -46,6 +46,8 @@ def lib():
             f.restype = ctypes.c_int
             f.argtypes = [_c_p] * 5 + [_c_i64] * 4 + [_c_p, _c_sz, _c_p]
         _c_i = ctypes.c_int
+        L.l1attn_dense_column_ranks_f32.restype = _c_i
+        L.l1attn_dense_column_ranks_f32.argtypes = [_c_p] * 4 + [_c_i64] * 4 + [_c_p]
         L.l1attn_expand_coo_workspace_bytes.restype = _c_sz
         L.l1attn_expand_coo_workspace_bytes.argtypes = [_c_i64]
         L.l1attn_expand_coo.restype = _c_i

@@ -10,15 +10,20 @@
 // (v_sub, v_add |x|) with no LDS or vector-memory traffic.  The workgroup (all heads of a 64-token
 // dst tile) transposes each finished src row through LDS and stores [t-tile x H] contiguous runs.
 //
-// Backward (fp32 fast path): one lane per (h,w) column, a workgroup per 32-token dst tile looping
-// over all src tokens.  q values and dq accumulators live in registers, the dA tile is staged
-// through LDS in [s][h][t] order so that a lane reads its head's four consecutive dA values with
-// one broadcast ds_read_b128.  Per pair-element: v_sub, v_med3 (sign with sign(0)=0), two v_fma.
+// Backward (fp32 fast path): one lane per (h,w) column, a workgroup per dst tile of 32..88 tokens
+// looping over all src tokens.  q values and dq accumulators live in registers, the dA tile is
+// staged through LDS in [s][h][t] order so that a lane reads its head's four consecutive dA values
+// with one broadcast ds_read_b128.  Per pair-element: v_sub, v_med3 (sign with sign(0)=0), two v_fma.
 // dq is complete when the loop ends; dk is written as one partial per dst tile and summed in
 // tile order by a second kernel, so the result is bitwise reproducible (no atomics).
+// For T >= 2048 the pair-element takes three instructions: q and k are first replaced by
+// order-preserving integer ranks per column (dense_rank.hip), on which a clamped subtraction is
+// already (sign+1)/2, and the row and column sums of dA turn the accumulated sums back into
+// sum(sign*dA).
 //
 // Generic kernels (any shape, float or double, exact comparisons) cover everything else.
 #include "common.h"
+#include "dense_rank.h"
 #include <math.h>
 #include <algorithm>
 
@@ -293,6 +298,22 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 constexpr int BWD_SJ = 4;  // src tokens per staging step
 constexpr float BWD_PRESCALE = 18446744073709551616.0f;  // 2^64
 
+// Sum over each aligned group of 16 lanes (a DPP row); the total lands in the group's last lane.
+// Lanes shifted in from outside the row read as zero.
+template <int CTRL>
+__device__ __forceinline__ float dpp_row_get(float x)
+{
+	return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_sum_to_last(float x)
+{
+	x += dpp_row_get<0x111>(x);  // row_shr:1
+	x += dpp_row_get<0x112>(x);  // row_shr:2
+	x += dpp_row_get<0x114>(x);  // row_shr:4
+	x += dpp_row_get<0x118>(x);  // row_shr:8
+	return x;
+}
+
 // sign(x) for pre-scaled differences: x is (q-k)*2^64, so every non-zero difference of
 // magnitude >= 2^-64 saturates to +-1 and an exact tie stays 0.
 //
@@ -324,6 +345,31 @@ __device__ __forceinline__ void pair_step4(const float* qc, float kc, const floa
 	    : "v"(qc[0]), "v"(qc[1]), "v"(qc[2]), "v"(qc[3]), "v"(kc), "v"(g.x), "v"(g.y), "v"(g.z), "v"(g.w));
 }
 
+// The same four pair-elements on column ranks (dense_rank.hip): qc holds rq, kc holds rk (rank minus
+// one half), so clamp(qc - kc, 0, 1) = hv is 1, 1/2 or 0 for q > k, q == k, q < k and sign = 2*hv - 1.
+//   dq_u += hv*g_u; dk += hv*g_u
+// Three instructions per pair-element; the caller turns the sums into sum(sign*g) with the row and
+// column sums of g:  sum_s sign*g = 2*sum_s hv*g - sum_s g.
+__device__ __forceinline__ void pair_step4_rank(const float* qc, float kc, const float4& g, float* dq, float& dk)
+{
+	float e0, e1;
+	asm volatile(
+	    "v_sub_f32_e64 %0, %7, %11 clamp\n\t"
+	    "v_sub_f32_e64 %1, %8, %11 clamp\n\t"
+	    "v_fmac_f32 %2, %0, %12\n\t"
+	    "v_fmac_f32 %6, %0, %12\n\t"
+	    "v_fmac_f32 %3, %1, %13\n\t"
+	    "v_fmac_f32 %6, %1, %13\n\t"
+	    "v_sub_f32_e64 %0, %9, %11 clamp\n\t"
+	    "v_sub_f32_e64 %1, %10, %11 clamp\n\t"
+	    "v_fmac_f32 %4, %0, %14\n\t"
+	    "v_fmac_f32 %6, %0, %14\n\t"
+	    "v_fmac_f32 %5, %1, %15\n\t"
+	    "v_fmac_f32 %6, %1, %15"
+	    : "=&v"(e0), "=&v"(e1), "+v"(dq[0]), "+v"(dq[1]), "+v"(dq[2]), "+v"(dq[3]), "+v"(dk)
+	    : "v"(qc[0]), "v"(qc[1]), "v"(qc[2]), "v"(qc[3]), "v"(kc), "v"(g.x), "v"(g.y), "v"(g.z), "v"(g.w));
+}
+
 // grid.x = dst tiles of tt_rows tokens, grid.y = column chunks of blockDim.x, grid.z = batches.
 // dkp: [n_ttiles][nb][T][HW] partials (or dk itself when there is a single dst tile).
 //
@@ -335,15 +381,25 @@ __device__ __forceinline__ void pair_step4(const float* qc, float kc, const floa
 // PER = staged dA values per thread and step (ceil(BWD_SJ*tt_rows*heads / blockDim.x) <= PER).  The dA
 // and k values of step n+1 are fetched into registers before the math of step n, so their latency
 // is covered by a whole step of VALU work.
-template <int TT, int MAXTHREADS, int PER>
+//
+// RANK: q and k point to the column ranks rq and rk (rank minus one half) and the pair-elements
+// take three instructions (pair_step4_rank).  The sums of g that turn sum(hv*g) into sum(sign*g)
+// come from the staged tile; they are read before the step's math and added up after the math of
+// its first src row, so that no wave waits for LDS: sixteen lanes per (src row, head) add up the
+// TT values and store the column sum to csp [n_ttiles][nb][T][H] (the reduction kernel needs it),
+// and every thread keeps the running sum over src rows of up to NR (head, dst token) slots (the
+// row sums that dq needs after the loop).  dkp then holds the raw sum(hv*g) partials.
+template <int TT, int MAXTHREADS, int PER, bool RANK>
 __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __restrict__ dA,
                                                                    const float* __restrict__ q,
                                                                    const float* __restrict__ k,
                                                                    float* __restrict__ dq, float* __restrict__ dkp,
-                                                                   int Tn, int H, int W, float scale)
+                                                                   float* __restrict__ csp, int Tn, int H, int W,
+                                                                   float scale)
 {
 	constexpr int TTP = TT + 4;  // LDS row pitch: keeps 16-byte alignment for ds_read_b128
 	constexpr int tt_rows = TT;
+	constexpr int NR = (PER + BWD_SJ - 1) / BWD_SJ;  // (head, dst token) slots per thread, >= HB*TT / blockDim.x
 	extern __shared__ float gl[];   // [BWD_SJ][HB][TTP]
 	const unsigned HW = (unsigned)(H * W);
 	const unsigned col0 = blockIdx.y * blockDim.x;
@@ -362,19 +418,21 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	const float* const k_b = k + (int64_t)b * Tn * HW;
 	const float* const dA_b = dA + ((int64_t)b * Tn * Tn + t0) * H + h_lo;
 	float* const dkp_b = dkp + ((int64_t)tt * nb + b) * Tn * HW;
+	float* const csp_b = RANK ? csp + ((int64_t)tt * nb + b) * Tn * H + h_lo : nullptr;
 
 	float qc[TT], dqa[TT];
 #pragma unroll
 	for (int i = 0; i < TT; i++) {
 		const int t = min(t0 + i, Tn - 1);
-		qc[i] = (q_b + (int64_t)t * HW)[col] * BWD_PRESCALE;
+		const float v = (q_b + (int64_t)t * HW)[col];
+		qc[i] = RANK ? v : v * BWD_PRESCALE;
 		dqa[i] = 0.0f;
 	}
 
 	// staging roles of this thread: element e = threadIdx.x + r*blockDim.x of the [j][i][hh] step tile
 	const int n_stage = BWD_SJ * tt_rows * HB;
 	int st_j[PER], st_lds[PER];
-	int64_t st_off[PER];
+	unsigned st_off[PER];  // within the step's BWD_SJ src rows of dA: below 2^31 (checked by the host)
 	bool st_ok[PER];
 #pragma unroll
 	for (int r = 0; r < PER; r++) {
@@ -383,15 +441,25 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		const int i = rr / HB, hh = rr % HB;
 		st_j[r] = j;
 		st_ok[r] = e < n_stage && t0 + i < Tn;
-		st_off[r] = ((int64_t)j * Tn + i) * H + hh;
+		st_off[r] = ((unsigned)j * (unsigned)Tn + (unsigned)i) * (unsigned)H + (unsigned)hh;
 		st_lds[r] = e < n_stage ? (j * HB + hh) * TTP + i : -1;
+	}
+	// RANK: row-sum slots of this thread, slot = hh*TT + i -> LDS offset hh*TTP + i of the j = 0 plane
+	int rs_lds[NR];
+	float rs_acc[NR];
+#pragma unroll
+	for (int n = 0; n < NR; n++) {
+		const int slot = threadIdx.x + n * blockDim.x;
+		rs_lds[n] = slot < HB * tt_rows ? (slot / tt_rows) * TTP + slot % tt_rows : -1;
+		rs_acc[n] = 0.0f;
 	}
 	float g_pre[PER], k_pre[BWD_SJ];
 	auto prefetch = [&](int s0) {
+		const float* const dA_s = dA_b + (int64_t)s0 * Tn * H;  // wave-uniform
 #pragma unroll
 		for (int r = 0; r < PER; r++) {
 			g_pre[r] = 0.0f;
-			if (st_ok[r] && s0 + st_j[r] < Tn) g_pre[r] = (dA_b + (int64_t)s0 * Tn * H)[st_off[r]];
+			if (st_ok[r] && s0 + st_j[r] < Tn) g_pre[r] = dA_s[st_off[r]];
 		}
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) k_pre[j] = (k_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
@@ -406,7 +474,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		float kc[BWD_SJ], dka[BWD_SJ];
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) {
-			kc[j] = k_pre[j] * BWD_PRESCALE;
+			kc[j] = RANK ? k_pre[j] : k_pre[j] * BWD_PRESCALE;
 			dka[j] = 0.0f;
 		}
 		lds_barrier();
@@ -416,6 +484,26 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			const float4* gp0 = reinterpret_cast<const float4*>(gl + hl * TTP);
 			constexpr int NI4 = TT / 4;
 			float4 g_cur = gp0[0];
+			// RANK: the tile values for the sums are read here and added up after the first src row's math,
+			// by which time they have arrived.  Column sums: row = jj*HB + hh of the tile, sixteen lanes per
+			// row (the host checks BWD_SJ*HB*16 <= blockDim.x).  Row sums: this thread's (head, dst token) slots.
+			constexpr int NM = (TT / 4 + 15) / 16;
+			const int cs_sub = threadIdx.x & 15, cs_row = threadIdx.x >> 4;
+			float4 cs_v[NM];
+			float rs_v[NR][BWD_SJ];
+			if (RANK) {
+				const float4* rp = reinterpret_cast<const float4*>(gl + cs_row * TTP);
+#pragma unroll
+				for (int m = 0; m < NM; m++) {
+					cs_v[m] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+					if (cs_row < BWD_SJ * HB && cs_sub + 16 * m < TT / 4) cs_v[m] = rp[cs_sub + 16 * m];
+				}
+#pragma unroll
+				for (int n = 0; n < NR; n++) {
+#pragma unroll
+					for (int jj = 0; jj < BWD_SJ; jj++) rs_v[n][jj] = rs_lds[n] >= 0 ? gl[jj * HB * TTP + rs_lds[n]] : 0.0f;
+				}
+			}
 #pragma unroll
 			for (int j = 0; j < BWD_SJ; j++) {
 #pragma unroll
@@ -424,7 +512,19 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 					if (i4 + 1 < NI4) g_nxt = gp0[(j * HB * TTP) / 4 + i4 + 1];
 					else if (j + 1 < BWD_SJ) g_nxt = gp0[((j + 1) * HB * TTP) / 4];
 					__builtin_amdgcn_sched_barrier(0);
-					pair_step4(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
+					if (RANK && j == 1 && i4 == 0) {
+						float a = 0.0f;
+#pragma unroll
+						for (int m = 0; m < NM; m++) a += (cs_v[m].x + cs_v[m].y) + (cs_v[m].z + cs_v[m].w);
+						a = row16_sum_to_last(a);
+						const int jj = cs_row / HB, s = s0 + jj;
+						if (cs_sub == 15 && cs_row < BWD_SJ * HB && s < Tn) csp_b[(int64_t)s * H + (cs_row - jj * HB)] = a;
+#pragma unroll
+						for (int n = 0; n < NR; n++) rs_acc[n] += (rs_v[n][0] + rs_v[n][1]) + (rs_v[n][2] + rs_v[n][3]);
+						__builtin_amdgcn_sched_barrier(0);
+					}
+					if (RANK) pair_step4_rank(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
+					else pair_step4(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
 					g_cur = g_nxt;
 				}
 			}
@@ -434,22 +534,56 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) {
 			const int s = s0 + j;
-			if (s < Tn) (dkp_b + (int64_t)s * HW)[col] = dka[j] * scale;
+			if (s < Tn) (dkp_b + (int64_t)s * HW)[col] = RANK ? dka[j] : dka[j] * scale;
 		}
 	}
 	float* const dq_b = dq + (int64_t)b * Tn * HW;
+	if (RANK) {
+		lds_barrier();  // the last step's tile reads are done
+		// exchange the row sums through the j = 0 plane of the tile: [hh][TTP]
 #pragma unroll
-	for (int i = 0; i < TT; i++) {
-		const int t = t0 + i;
-		if (t < Tn) (dq_b + (int64_t)t * HW)[col] = dqa[i] * scale;
+		for (int n = 0; n < NR; n++)
+			if (rs_lds[n] >= 0) gl[rs_lds[n]] = rs_acc[n];
+		lds_barrier();
+		const float4* rp = reinterpret_cast<const float4*>(gl + hl * TTP);
+#pragma unroll
+		for (int i4 = 0; i4 < TT / 4; i4++) {
+			const float4 r4 = rp[i4];
+			const float rr[4] = {r4.x, r4.y, r4.z, r4.w};
+#pragma unroll
+			for (int u = 0; u < 4; u++) {
+				const int t = t0 + i4 * 4 + u;
+				if (t < Tn) (dq_b + (int64_t)t * HW)[col] = (2.0f * dqa[i4 * 4 + u] - rr[u]) * scale;
+			}
+		}
+	} else {
+#pragma unroll
+		for (int i = 0; i < TT; i++) {
+			const int t = t0 + i;
+			if (t < Tn) (dq_b + (int64_t)t * HW)[col] = dqa[i] * scale;
+		}
 	}
 }
 
+// One (b, s, h) element per thread: the column sums of all dst tiles, in tile order.
+__global__ __launch_bounds__(256) void dense_bwd_reduce_colsum(const float* __restrict__ csp, float* __restrict__ cs,
+                                                                 int64_t n, int n_tt)
+{
+	const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (i >= n) return;
+	float acc = csp[i];
+	for (int tt = 1; tt < n_tt; tt++) acc += csp[(int64_t)tt * n + i];
+	cs[i] = acc;
+}
+
 // dk[i] = sum over dst tiles, in tile order, of the partials; n = nb*T*HW elements per tile.
-// VEC: n and both base pointers are multiples of 4 floats.
-template <bool VEC>
+// VEC: n and both base pointers are multiples of 4 floats (RANK: and so is W).
+// RANK: the partials are sums of hv*g; with the column sums cs [nb][T][H] of g,
+//   dk = scale * (cs - 2 * sum of partials).
+template <bool VEC, bool RANK>
 __global__ __launch_bounds__(256) void dense_bwd_reduce_dk(const float* __restrict__ dkp, float* __restrict__ dk,
-                                                             int64_t n, int n_tt)
+                                                             int64_t n, int n_tt, const float* __restrict__ cs,
+                                                             int HW, int W, int H, float scale)
 {
 	if (VEC) {
 		const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
@@ -459,12 +593,18 @@ __global__ __launch_bounds__(256) void dense_bwd_reduce_dk(const float* __restri
 			const float4 p = *reinterpret_cast<const float4*>(dkp + (int64_t)tt * n + i);
 			acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
 		}
+		if (RANK) {
+			const float c = cs[(i / HW) * H + (int)(i % HW) / W];
+			acc.x = (c - 2.0f * acc.x) * scale; acc.y = (c - 2.0f * acc.y) * scale;
+			acc.z = (c - 2.0f * acc.z) * scale; acc.w = (c - 2.0f * acc.w) * scale;
+		}
 		*reinterpret_cast<float4*>(dk + i) = acc;
 	} else {
 		const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
 		if (i >= n) return;
 		float acc = dkp[i];
 		for (int tt = 1; tt < n_tt; tt++) acc += dkp[(int64_t)tt * n + i];
+		if (RANK) acc = (cs[(i / HW) * H + (int)(i % HW) / W] - 2.0f * acc) * scale;
 		dk[i] = acc;
 	}
 }
@@ -558,10 +698,13 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 
 struct BwdPlan {
 	bool fast;
-	bool wide;        // TTMAX 96 / 512-thread instantiation
+	bool wide;        // TT 64..88 / 512-thread instantiation
+	bool rank;        // three-instruction pair-elements on column ranks
 	int threads, n_cc, n_tt, tt_rows, per;
 	size_t lds_bytes;
-	size_t per_batch_bytes;  // partial-dk scratch for one batch (0 when a single dst tile)
+	size_t partial_bytes;    // partial-dk scratch for one batch (0 when a single dst tile)
+	size_t rank_bytes;       // rq and rk of one batch (0 unless rank)
+	size_t per_batch_bytes;  // workspace share of one batch
 };
 
 constexpr int N_CU = 256;
@@ -570,51 +713,77 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 {
 	BwdPlan p{};
 	const int64_t HW = H * W;
-	p.fast = B >= 1 && T >= 16 && HW >= 32 && T <= (1 << 30) && B <= 65535 && HW <= (int64_t)512 * 65535;
+	p.fast = B >= 1 && T >= 16 && HW >= 32 && T <= (1 << 30) && B <= 65535 && HW <= (int64_t)512 * 65535 &&
+	         (BWD_SJ * T + 128) * H < ((int64_t)1 << 31);  // 32-bit staging offsets
 	if (!p.fast) return p;
 	// wide tiles pay off once there are enough dst tokens to give every CU a few workgroups
 	p.wide = T >= 1024 && B * l1_cdiv(HW, 512) * l1_cdiv(T, 88) >= N_CU;
 	const int maxthreads = p.wide ? 512 : 1024;
 	p.threads = (int)std::min<int64_t>(maxthreads, l1_cdiv(HW, 64) * 64);
 	p.n_cc = (int)l1_cdiv(HW, p.threads);
+	int64_t hb_exact = 1;  // most heads any column chunk touches
+	for (int64_t cc = 0; cc < p.n_cc; cc++) {
+		const int64_t c0 = cc * p.threads, c1 = std::min<int64_t>(HW, c0 + p.threads) - 1;
+		hb_exact = std::max<int64_t>(hb_exact, c1 / W - c0 / W + 1);
+	}
+	// The rank transform costs O(T log T) per column against O(T^2) saved instructions: it pays off for
+	// long sequences, and one workgroup must be able to sort a column in LDS.
+	// Its column sums use sixteen lanes per (src row, head) of a step.
+	p.rank = p.wide && T >= 2048 && l1_column_ranks_ok(B, T, H, W) && BWD_SJ * hb_exact * 16 <= p.threads;
 	p.tt_rows = p.wide ? 88 : 32;
 	if (p.wide) {
 		// one workgroup per CU at a time: pick the tile height that wastes the least of the last round
 		double best = 1e30;
-		for (int tr = 64; tr <= 88; tr += 8) {
+		const int tr_max = p.rank ? 80 : 88;  // the rank variant keeps a few more values in registers
+		for (int tr = 64; tr <= tr_max; tr += 8) {
 			const int64_t wgs = B * p.n_cc * l1_cdiv(T, tr);
 			const double cost = (double)l1_cdiv(wgs, N_CU) * tr * (1.0 + 3.0 / tr);  // rounds x rows, plus partial traffic
 			if (cost < best) { best = cost; p.tt_rows = tr; }
 		}
 	}
 	p.n_tt = (int)l1_cdiv(T, p.tt_rows);
-	const int64_t hb_max = std::min<int64_t>(H, (p.threads + W - 2) / W + 1);
+	const int64_t hb_max = hb_exact;
 	p.lds_bytes = (size_t)BWD_SJ * hb_max * (p.tt_rows + 4) * sizeof(float);
 	p.per = (int)l1_cdiv((int64_t)BWD_SJ * p.tt_rows * hb_max, p.threads);
 	if (p.lds_bytes > 64 * 1024 || p.per > 16 || (p.wide && p.per > 8)) { p.fast = false; return p; }
-	p.per_batch_bytes = p.n_tt > 1 ? (size_t)p.n_tt * T * HW * sizeof(float) : 0;
+	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_tt * T * HW * sizeof(float) : 0;
+	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
+	p.rank_bytes = p.rank ? ((size_t)2 * T * HW + (size_t)(p.n_tt + 1) * T * H) * sizeof(float) : 0;
+	p.per_batch_bytes = p.partial_bytes + p.rank_bytes;
 	return p;
 }
 
 void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* dA, const float* q, const float* k,
-                     float* dq, float* dkp, int T, int H, int W, float scale)
+                     float* dq, float* dkp, float* csp, int T, int H, int W, float scale)
 {
-#define L1_BWD_CASE(TTV, MT, PERV)                                                                              \
-	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV>), grid, dim3(p.threads), p.lds_bytes, st, dA, q, k, dq,   \
-	                   dkp, T, H, W, scale)
-	if (p.wide) {
+#define L1_BWD_CASE(TTV, MT, PERV, RANKV)                                                                       \
+	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV, RANKV>), grid, dim3(p.threads), p.lds_bytes, st, dA, q,   \
+	                   k, dq, dkp, csp, T, H, W, scale)
+	if (p.wide && p.rank) {
 		switch (p.tt_rows) {
-		case 64: L1_BWD_CASE(64, 512, 8); break;
-		case 72: L1_BWD_CASE(72, 512, 8); break;
-		case 80: L1_BWD_CASE(80, 512, 8); break;
-		default: L1_BWD_CASE(88, 512, 8); break;
+		case 64:
+			if (p.per <= 4) L1_BWD_CASE(64, 512, 4, true);
+			else L1_BWD_CASE(64, 512, 8, true);
+			break;
+		case 72: L1_BWD_CASE(72, 512, 8, true); break;
+		default: L1_BWD_CASE(80, 512, 8, true); break;
+		}
+	} else if (p.wide) {
+		switch (p.tt_rows) {
+		case 64:
+			if (p.per <= 4) L1_BWD_CASE(64, 512, 4, false);
+			else L1_BWD_CASE(64, 512, 8, false);
+			break;
+		case 72: L1_BWD_CASE(72, 512, 8, false); break;
+		case 80: L1_BWD_CASE(80, 512, 8, false); break;
+		default: L1_BWD_CASE(88, 512, 8, false); break;
 		}
 	} else {
-		if (p.per <= 1) L1_BWD_CASE(32, 1024, 1);
-		else if (p.per <= 2) L1_BWD_CASE(32, 1024, 2);
-		else if (p.per <= 4) L1_BWD_CASE(32, 1024, 4);
-		else if (p.per <= 8) L1_BWD_CASE(32, 1024, 8);
-		else L1_BWD_CASE(32, 1024, 16);
+		if (p.per <= 1) L1_BWD_CASE(32, 1024, 1, false);
+		else if (p.per <= 2) L1_BWD_CASE(32, 1024, 2, false);
+		else if (p.per <= 4) L1_BWD_CASE(32, 1024, 4, false);
+		else if (p.per <= 8) L1_BWD_CASE(32, 1024, 8, false);
+		else L1_BWD_CASE(32, 1024, 16, false);
 	}
 #undef L1_BWD_CASE
 }
@@ -671,28 +840,52 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 	const int64_t HW = H * W;
 	if (p.per_batch_bytes == 0) {
 		dim3 grid(1, p.n_cc, (unsigned)B);
-		launch_bwd_fast(p, grid, st, d_attn, q, k, dq, dk, (int)T, (int)H, (int)W, scale);
+		launch_bwd_fast(p, grid, st, d_attn, q, k, dq, dk, nullptr, (int)T, (int)H, (int)W, scale);
 		L1_LAUNCH_CHECK();
 		return L1ATTN_OK;
 	}
 	if (!workspace || workspace_bytes < p.per_batch_bytes) return L1ATTN_ERR_WORKSPACE;
 	int64_t nb_max = (int64_t)(workspace_bytes / p.per_batch_bytes);
 	if (nb_max > B) nb_max = B;
+	// workspace: [n_tt][nb_max][T][HW] dk partials, then (rank path) rq and rk [nb_max][T][HW] each, the
+	// column sums per dst tile [n_tt][nb_max][T][H] and their total [nb_max][T][H]
 	float* dkp = (float*)workspace;
+	float* rq = dkp + (size_t)nb_max * (p.partial_bytes / sizeof(float));
+	float* rk = rq + (size_t)nb_max * T * HW;
+	float* csp = rk + (size_t)nb_max * T * HW;
+	float* cs = csp + (size_t)p.n_tt * nb_max * T * H;
 	for (int64_t b0 = 0; b0 < B; b0 += nb_max) {
 		const int64_t nb = std::min<int64_t>(nb_max, B - b0);
 		dim3 grid(p.n_tt, p.n_cc, (unsigned)nb);
-		launch_bwd_fast(p, grid, st, d_attn + b0 * T * T * H, q + b0 * T * HW, k + b0 * T * HW, dq + b0 * T * HW, dkp,
-		                (int)T, (int)H, (int)W, scale);
+		const float* qa = q + b0 * T * HW;
+		const float* ka = k + b0 * T * HW;
+		if (p.rank) {
+			const int rc = l1_launch_column_ranks(qa, ka, rq, rk, nb, T, H, W, st);
+			if (rc != L1ATTN_OK) return rc;
+			qa = rq;
+			ka = rk;
+		}
+		launch_bwd_fast(p, grid, st, d_attn + b0 * T * T * H, qa, ka, dq + b0 * T * HW, dkp, csp, (int)T, (int)H,
+		                (int)W, scale);
 		L1_LAUNCH_CHECK();
 		const int64_t ne = nb * T * HW;
-		const bool vec = ((T * HW) % 4 == 0) && ((((uintptr_t)dkp) | ((uintptr_t)dk)) & 15) == 0;
-		if (vec)
-			hipLaunchKernelGGL(dense_bwd_reduce_dk<true>, dim3((unsigned)l1_cdiv(ne, 1024)), dim3(256), 0, st, dkp,
-			                   dk + b0 * T * HW, ne, p.n_tt);
-		else
-			hipLaunchKernelGGL(dense_bwd_reduce_dk<false>, dim3((unsigned)l1_cdiv(ne, 256)), dim3(256), 0, st, dkp,
-			                   dk + b0 * T * HW, ne, p.n_tt);
+		if (p.rank) {
+			const int64_t nc = nb * T * H;
+			hipLaunchKernelGGL(dense_bwd_reduce_colsum, dim3((unsigned)l1_cdiv(nc, 256)), dim3(256), 0, st, csp, cs, nc,
+			                   p.n_tt);
+			L1_LAUNCH_CHECK();
+		}
+		const bool vec = ((T * HW) % 4 == 0) && ((((uintptr_t)dkp) | ((uintptr_t)dk)) & 15) == 0 &&
+		                 (!p.rank || W % 4 == 0);
+		const dim3 rgrid((unsigned)l1_cdiv(ne, vec ? 1024 : 256));
+#define L1_REDUCE_CASE(VECV, RANKV)                                                                             \
+	hipLaunchKernelGGL((dense_bwd_reduce_dk<VECV, RANKV>), rgrid, dim3(256), 0, st, dkp, dk + b0 * T * HW, ne,    \
+	                   p.n_tt, cs, (int)HW, (int)W, (int)H, scale)
+		if (vec && p.rank) L1_REDUCE_CASE(true, true);
+		else if (vec) L1_REDUCE_CASE(true, false);
+		else if (p.rank) L1_REDUCE_CASE(false, true);
+		else L1_REDUCE_CASE(false, false);
+#undef L1_REDUCE_CASE
 		L1_LAUNCH_CHECK();
 	}
 	return L1ATTN_OK;

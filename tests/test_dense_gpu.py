@@ -163,6 +163,103 @@ def test_dense_mid_size_vs_closed_form():
         assert cf.rel_err(kd.grad[b:b + 1], k64.grad) <= BWD_TOL
 
 
+def _with_ties(q, k, seed):
+    """Plant exact ties: dst rows copied from src rows, a zero column with both signs of zero,
+    and a column quantised to a few values (many equal pairs)."""
+    g = torch.Generator().manual_seed(seed)
+    T = q.shape[1]
+    idx = torch.randperm(T, generator=g)[: T // 8]
+    q[:, idx] = k[:, idx.flip(0)]
+    q[..., 0] = 0.0
+    k[..., 0] = -0.0
+    q[..., 1] = torch.round(q[..., 1])
+    k[..., 1] = torch.round(k[..., 1])
+    return q, k
+
+
+@pytest.mark.parametrize("shape,tag", [((6, 1024, 32, 64), "wide tiles, sign from the scaled difference"),
+                                       ((3, 2048, 32, 64), "wide tiles, sign from column ranks")])
+def test_dense_backward_long_sequences_vs_oracle(shape, tag):
+    """The two backward paths for long sequences (dst tiles of 64..88 tokens; for T >= 2048 on column
+    ranks), with planted ties, against the oracle."""
+    B, T, H, W = shape
+    print("case dense long", shape, tag, flush=True)
+    q, k, da = _inputs(B, T, H, W, seed=77 + T)
+    q, k = _with_ties(q, k, seed=T)
+    import _l1attn_hip as drv
+    dq, dk = drv.dense_backward(da.cuda(), q.cuda(), k.cuda())
+    torch.cuda.synchronize()
+    rdq, rdk = oracle.dense_bwd(da.double(), q.double(), k.double())
+    assert cf.rel_err(dq.cpu(), rdq) <= BWD_TOL
+    assert cf.rel_err(dk.cpu(), rdk) <= BWD_TOL
+    # the planted all-tie column gets no gradient (on ranks the two halves of the sum cancel up to
+    # fp32 rounding of sums of T terms)
+    tie_dq = float(dq[..., 0].abs().max()) / float(rdq.abs().max())
+    tie_dk = float(dk[..., 0].abs().max()) / float(rdk.abs().max())
+    assert tie_dq <= 1e-5 and tie_dk <= 1e-5
+
+
+def test_dense_column_ranks():
+    """First stage of the long-sequence backward: the rank maps keep order and ties of every column."""
+    import ctypes
+    import _l1attn_hip as drv
+    L = drv.lib()
+    for (B, T, H, W), seed in [((2, 64, 2, 8), 1), ((1, 513, 2, 3), 2), ((1, 2048, 1, 4), 3)]:
+        print("case dense ranks", (B, T, H, W), flush=True)
+        q, k, _ = _inputs(B, T, H, W, seed=seed)
+        q, k = _with_ties(q, k, seed)
+        qd, kd = q.cuda(), k.cuda()
+        rq, rk = torch.empty_like(qd), torch.empty_like(kd)
+        rc = L.l1attn_dense_column_ranks_f32(drv.ptr(qd), drv.ptr(kd), drv.ptr(rq), drv.ptr(rk), B, T, H, W,
+                                             drv.stream_of(qd))
+        assert rc == 0
+        torch.cuda.synchronize()
+        for t0 in range(0, T, 256):  # all (t, s) pairs, a slab of dst tokens at a time
+            d = rq[:, t0:t0 + 256, None] - (rk[:, None] + 0.5)
+            ref = torch.sign(qd[:, t0:t0 + 256, None] - kd[:, None])
+            assert torch.equal(torch.clamp(d, -1, 1), ref)
+            assert torch.equal(2 * torch.clamp(d + 0.5, 0, 1) - 1, ref)
+        assert float(rq.min()) >= -1 and float(rq.max()) <= 2 * T and float(rk.min()) >= -0.5
+    too_long = torch.zeros(1, 8193, 1, 1).cuda()
+    out = torch.empty_like(too_long)
+    assert L.l1attn_dense_column_ranks_f32(drv.ptr(too_long), drv.ptr(too_long), drv.ptr(out), drv.ptr(out),
+                                           1, 8193, 1, 1, drv.stream_of(too_long)) == -3
+
+
+def test_dense_headline_size_properties():
+    """BASELINE config 3 (B=8, T=4096, H=16, W=64), where the loop oracle would take an hour:
+    sampled rows of A, dq and dk against the defining sums in fp64, the checksum
+    sum_t dq[b,t,h,w] = -sum_s dk[b,s,h,w], and bitwise repeatability."""
+    print("case dense headline size", flush=True)
+    B, T, H, W = 8, 4096, 16, 64
+    g = torch.Generator(device="cuda").manual_seed(4096)
+    q = torch.randn(B, T, H, W, generator=g, device="cuda")
+    k = torch.randn(B, T, H, W, generator=g, device="cuda")
+    q[:, 5] = k[:, 9]            # exact ties at full size
+    q[..., 3] = torch.round(q[..., 3] * 2) / 2
+    k[..., 3] = torch.round(k[..., 3] * 2) / 2
+    da = torch.randn(B, T, T, H, generator=g, device="cuda")
+    import _l1attn_hip as drv
+    a = drv.dense_forward(q, k)[0]
+    dq, dk = drv.dense_backward(da, q, k)
+    dq2, dk2 = drv.dense_backward(da, q, k)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2)
+    scale = -1.0 / math.sqrt(W)
+    q64, k64 = q.double(), k.double()
+    for b, r in [(0, 0), (3, 5), (7, 4095), (5, 2049)]:
+        # row r as dst token: A[b,:,r,:] and dq[b,r]; row r as src token: dk[b,r]
+        diff = q64[b, r][None] - k64[b]                                   # [S,H,W]
+        ra = scale * diff.abs().sum(-1)
+        assert cf.rel_err(a[b, :, r, :].cpu(), ra.cpu()) <= FWD_TOL
+        rdq = scale * (torch.sign(diff) * da[b, :, r, :, None].double()).sum(0)
+        assert cf.rel_err(dq[b, r].cpu(), rdq.cpu()) <= BWD_TOL
+        diff = q64[b] - k64[b, r][None]                                   # [T,H,W]
+        rdk = -scale * (torch.sign(diff) * da[b, r, :, :, None].double()).sum(0)
+        assert cf.rel_err(dk[b, r].cpu(), rdk.cpu()) <= BWD_TOL
+    sq, sk = dq.double().sum(1), dk.double().sum(1)
+    assert float((sq + sk).abs().max()) <= 1e-4 * float(sq.abs().max())
+
+
 def test_dense_input_checks():
     m = _mods()
     import _l1attn_hip as drv
