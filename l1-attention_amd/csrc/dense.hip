@@ -389,13 +389,13 @@ __device__ __forceinline__ void pair_step4_rank(const float* qc, float kc, const
 // TT values and store the column sum to csp [n_ttiles][nb][T][H] (the reduction kernel needs it),
 // and every thread keeps the running sum over src rows of up to NR (head, dst token) slots (the
 // row sums that dq needs after the loop).  dkp then holds the raw sum(hv*g) partials.
-template <int TT, int MAXTHREADS, int PER, bool RANK>
+template <int TT, int MAXTHREADS, int PER, bool RANK, bool GROUPED, bool FAST>
 __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __restrict__ dA,
                                                                    const float* __restrict__ q,
                                                                    const float* __restrict__ k,
                                                                    float* __restrict__ dq, float* __restrict__ dkp,
                                                                    float* __restrict__ csp, int Tn, int H, int W,
-                                                                   float scale)
+                                                                   float scale, int G)
 {
 	constexpr int TTP = TT + 4;  // LDS row pitch: keeps 16-byte alignment for ds_read_b128
 	constexpr int tt_rows = TT;
@@ -412,12 +412,19 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	const int HB = (int)(col_end / (unsigned)W) - h_lo + 1;  // heads this workgroup touches
 	const int hl = (int)(col / (unsigned)W) - h_lo;
 	const int b = blockIdx.z, nb = gridDim.z;
-	const int tt = blockIdx.x, t0 = tt * tt_rows;
 	// wave-uniform row bases; lanes add the 32-bit column
 	const float* const q_b = q + (int64_t)b * Tn * HW;
 	const float* const k_b = k + (int64_t)b * Tn * HW;
+	float* const dkp_b = dkp + ((int64_t)blockIdx.x * nb + b) * Tn * HW;
+	// GROUPED: the workgroup takes G consecutive dst tiles one after the other and keeps one dk partial
+	// for all of them: from the second tile on, a step adds to what the earlier tiles stored (same lane,
+	// same address, in tile order), which cuts the partial arrays and the reduction G-fold.
+	const int n_sub = GROUPED ? G : 1;
+#pragma nounroll
+	for (int u = 0; u < n_sub; u++) {
+	const int tt = blockIdx.x * n_sub + u, t0 = tt * tt_rows;
+	if (t0 >= Tn) break;
 	const float* const dA_b = dA + ((int64_t)b * Tn * Tn + t0) * H + h_lo;
-	float* const dkp_b = dkp + ((int64_t)tt * nb + b) * Tn * HW;
 	float* const csp_b = RANK ? csp + ((int64_t)tt * nb + b) * Tn * H + h_lo : nullptr;
 
 	float qc[TT], dqa[TT];
@@ -454,23 +461,52 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		rs_acc[n] = 0.0f;
 	}
 	float g_pre[PER], k_pre[BWD_SJ];
+	// interior tile with every staging role in use: the loads and LDS writes need no per-lane predicates.
+	// FAST: the host found this to hold for every workgroup of the launch, T a multiple of BWD_SJ and no
+	// idle lanes; the step loop is then compiled without a single branch around a memory access (the
+	// branches of the general form cost about 4 % of the kernel).
+	const bool full = FAST || (t0 + tt_rows <= Tn && n_stage == PER * (int)blockDim.x);
+	// loads of the dA and k values of the step that starts at src token s0
 	auto prefetch = [&](int s0) {
 		const float* const dA_s = dA_b + (int64_t)s0 * Tn * H;  // wave-uniform
+		if (FAST || (full && s0 + BWD_SJ <= Tn)) {
 #pragma unroll
-		for (int r = 0; r < PER; r++) {
-			g_pre[r] = 0.0f;
-			if (st_ok[r] && s0 + st_j[r] < Tn) g_pre[r] = dA_s[st_off[r]];
+			for (int r = 0; r < PER; r++) g_pre[r] = dA_s[st_off[r]];
+		} else {
+#pragma unroll
+			for (int r = 0; r < PER; r++) {
+				g_pre[r] = 0.0f;
+				if (st_ok[r] && s0 + st_j[r] < Tn) g_pre[r] = dA_s[st_off[r]];
+			}
 		}
 #pragma unroll
-		for (int j = 0; j < BWD_SJ; j++) k_pre[j] = (k_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
+		for (int j = 0; j < BWD_SJ; j++)
+			k_pre[j] = (k_b + (int64_t)(FAST ? s0 + j : min(s0 + j, Tn - 1)) * HW)[col];
+	};
+	// Wait for the prefetched values.  Loads and stores share one counter and may complete out of
+	// order, so a wait for a load while a store is in flight is a wait for everything.  The values
+	// are therefore taken before a step's stores are issued (the loads are a whole step old by then),
+	// and before the loop for the first step: otherwise each step's first use of them also waits for
+	// the previous step's stores to be acknowledged.
+	auto settle = [&]() {
+#pragma unroll
+		for (int r = 0; r < PER; r++) asm volatile("" : "+v"(g_pre[r]));
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) asm volatile("" : "+v"(k_pre[j]));
 	};
 	prefetch(0);
+	settle();
 
 	for (int s0 = 0; s0 < Tn; s0 += BWD_SJ) {
 		lds_barrier();  // the previous step's LDS reads are done
+		if (full) {
 #pragma unroll
-		for (int r = 0; r < PER; r++)
-			if (st_lds[r] >= 0) gl[st_lds[r]] = g_pre[r];
+			for (int r = 0; r < PER; r++) gl[st_lds[r]] = g_pre[r];
+		} else {
+#pragma unroll
+			for (int r = 0; r < PER; r++)
+				if (st_lds[r] >= 0) gl[st_lds[r]] = g_pre[r];
+		}
 		float kc[BWD_SJ], dka[BWD_SJ];
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) {
@@ -478,7 +514,23 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			dka[j] = 0.0f;
 		}
 		lds_barrier();
-		if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
+		// next step's values; FAST: the last step reads the last rows again, and nobody uses them
+		if (FAST) prefetch(min(s0 + BWD_SJ, Tn - BWD_SJ));
+		else if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
+		// what the earlier tiles of this workgroup left in the partial rows of this step; used after the math
+		float dk_old[BWD_SJ];
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) dk_old[j] = 0.0f;
+		if (GROUPED && FAST) {
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) {
+				const float o = (dkp_b + (int64_t)(s0 + j) * HW)[col];  // first tile: not written yet, not used
+				dk_old[j] = u > 0 ? o : 0.0f;
+			}
+		} else if (GROUPED && u > 0) {
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) dk_old[j] = (dkp_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
+		}
 		{
 			// all dA values of this step for the lane's head, read one float4 ahead of their use
 			const float4* gp0 = reinterpret_cast<const float4*>(gl + hl * TTP);
@@ -513,12 +565,22 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 					else if (j + 1 < BWD_SJ) g_nxt = gp0[((j + 1) * HB * TTP) / 4];
 					__builtin_amdgcn_sched_barrier(0);
 					if (RANK && j == 1 && i4 == 0) {
+						// keep the loaded values opaque up to here, or the adds (and the wait for the loads)
+						// are hoisted in front of the first src row's math
+#pragma unroll
+						for (int m = 0; m < NM; m++)
+							asm volatile("" : "+v"(cs_v[m].x), "+v"(cs_v[m].y), "+v"(cs_v[m].z), "+v"(cs_v[m].w));
+#pragma unroll
+						for (int n = 0; n < NR; n++) {
+#pragma unroll
+							for (int jj = 0; jj < BWD_SJ; jj++) asm volatile("" : "+v"(rs_v[n][jj]));
+						}
 						float a = 0.0f;
 #pragma unroll
 						for (int m = 0; m < NM; m++) a += (cs_v[m].x + cs_v[m].y) + (cs_v[m].z + cs_v[m].w);
 						a = row16_sum_to_last(a);
 						const int jj = cs_row / HB, s = s0 + jj;
-						if (cs_sub == 15 && cs_row < BWD_SJ * HB && s < Tn) csp_b[(int64_t)s * H + (cs_row - jj * HB)] = a;
+						if (cs_sub == 15 && cs_row < BWD_SJ * HB && (FAST || s < Tn)) csp_b[(int64_t)s * H + (cs_row - jj * HB)] = a;
 #pragma unroll
 						for (int n = 0; n < NR; n++) rs_acc[n] += (rs_v[n][0] + rs_v[n][1]) + (rs_v[n][2] + rs_v[n][3]);
 						__builtin_amdgcn_sched_barrier(0);
@@ -529,12 +591,14 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 				}
 			}
 		}
+		settle();
 		// unconditional in the lane dimension: a store guarded by a per-lane predicate would let the
 		// compiler sink the dk chain into the guarded block and split the four-instruction groups
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) {
 			const int s = s0 + j;
-			if (s < Tn) (dkp_b + (int64_t)s * HW)[col] = RANK ? dka[j] : dka[j] * scale;
+			const float v = RANK ? dka[j] : dka[j] * scale;
+			if (FAST || s < Tn) (dkp_b + (int64_t)s * HW)[col] = GROUPED ? dk_old[j] + v : v;
 		}
 	}
 	float* const dq_b = dq + (int64_t)b * Tn * HW;
@@ -553,16 +617,17 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 #pragma unroll
 			for (int u = 0; u < 4; u++) {
 				const int t = t0 + i4 * 4 + u;
-				if (t < Tn) (dq_b + (int64_t)t * HW)[col] = (2.0f * dqa[i4 * 4 + u] - rr[u]) * scale;
+				if (FAST || t < Tn) (dq_b + (int64_t)t * HW)[col] = (2.0f * dqa[i4 * 4 + u] - rr[u]) * scale;
 			}
 		}
 	} else {
 #pragma unroll
 		for (int i = 0; i < TT; i++) {
 			const int t = t0 + i;
-			if (t < Tn) (dq_b + (int64_t)t * HW)[col] = dqa[i] * scale;
+			if (FAST || t < Tn) (dq_b + (int64_t)t * HW)[col] = dqa[i] * scale;
 		}
 	}
+	}  // dst tiles of the workgroup
 }
 
 // One (b, s, h) element per thread: the column sums of all dst tiles, in tile order.
@@ -701,6 +766,8 @@ struct BwdPlan {
 	bool wide;        // TT 64..88 / 512-thread instantiation
 	bool rank;        // three-instruction pair-elements on column ranks
 	int threads, n_cc, n_tt, tt_rows, per;
+	bool branch_free;        // every workgroup of the launch runs whole tiles and whole steps
+	int group, n_groups;     // consecutive dst tiles per workgroup (sharing one dk partial); workgroups along T
 	size_t lds_bytes;
 	size_t partial_bytes;    // partial-dk scratch for one batch (0 when a single dst tile)
 	size_t rank_bytes;       // rq and rk of one batch (0 unless rank)
@@ -731,22 +798,34 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	// Its column sums use sixteen lanes per (src row, head) of a step.
 	p.rank = p.wide && T >= 2048 && l1_column_ranks_ok(B, T, H, W) && BWD_SJ * hb_exact * 16 <= p.threads;
 	p.tt_rows = p.wide ? 88 : 32;
+	p.group = 1;
 	if (p.wide) {
-		// one workgroup per CU at a time: pick the tile height that wastes the least of the last round
+		// One workgroup per CU at a time.  Pick the tile height and the tiles per workgroup that waste the
+		// least of the last round of workgroups; every partial array costs a write in the main kernel and
+		// a read in the reduction (0.04 tile rows per array, batch and column chunk, measured).
 		double best = 1e30;
 		const int tr_max = p.rank ? 80 : 88;  // the rank variant keeps a few more values in registers
 		for (int tr = 64; tr <= tr_max; tr += 8) {
-			const int64_t wgs = B * p.n_cc * l1_cdiv(T, tr);
-			const double cost = (double)l1_cdiv(wgs, N_CU) * tr * (1.0 + 3.0 / tr);  // rounds x rows, plus partial traffic
-			if (cost < best) { best = cost; p.tt_rows = tr; }
+			for (int g = 1; g <= 8; g *= 2) {
+				const int64_t ngr = l1_cdiv(l1_cdiv(T, tr), g);
+				const int64_t wgs = B * p.n_cc * ngr;
+				// tiles are grouped only in the 64-token instantiations (registers), see launch_bwd_fast()
+				const int64_t per_tr = l1_cdiv((int64_t)BWD_SJ * tr * hb_exact, p.threads);
+				if (g > 1 && (wgs < N_CU || tr != 64 || per_tr > (p.rank ? 4 : 8))) continue;
+				const double cost = (double)l1_cdiv(wgs, N_CU) * g * (tr + 1.0) + 0.04 * (double)(B * p.n_cc * ngr);
+				if (cost < best) { best = cost; p.tt_rows = tr; p.group = g; }
+			}
 		}
 	}
 	p.n_tt = (int)l1_cdiv(T, p.tt_rows);
+	p.n_groups = (int)l1_cdiv(p.n_tt, p.group);
 	const int64_t hb_max = hb_exact;
 	p.lds_bytes = (size_t)BWD_SJ * hb_max * (p.tt_rows + 4) * sizeof(float);
 	p.per = (int)l1_cdiv((int64_t)BWD_SJ * p.tt_rows * hb_max, p.threads);
 	if (p.lds_bytes > 64 * 1024 || p.per > 16 || (p.wide && p.per > 8)) { p.fast = false; return p; }
-	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_tt * T * HW * sizeof(float) : 0;
+	p.branch_free = p.wide && p.tt_rows == 64 && T % 64 == 0 && T % BWD_SJ == 0 && HW % p.threads == 0 &&
+	                p.threads % W == 0 && (int64_t)BWD_SJ * 64 * (p.threads / W) == (int64_t)4 * p.threads;
+	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_groups * T * HW * sizeof(float) : 0;
 	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
 	p.rank_bytes = p.rank ? ((size_t)2 * T * HW + (size_t)(p.n_tt + 1) * T * H) * sizeof(float) : 0;
 	p.per_batch_bytes = p.partial_bytes + p.rank_bytes;
@@ -756,36 +835,49 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* dA, const float* q, const float* k,
                      float* dq, float* dkp, float* csp, int T, int H, int W, float scale)
 {
-#define L1_BWD_CASE(TTV, MT, PERV, RANKV)                                                                       \
-	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV, RANKV>), grid, dim3(p.threads), p.lds_bytes, st, dA, q,   \
-	                   k, dq, dkp, csp, T, H, W, scale)
-	if (p.wide && p.rank) {
+#define L1_BWD_CASE6(TTV, MT, PERV, RANKV, GRPV, FASTV)                                                         \
+	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV, RANKV, GRPV, FASTV>), grid, dim3(p.threads), p.lds_bytes, \
+	                   st, dA, q, k, dq, dkp, csp, T, H, W, scale, p.group)
+#define L1_BWD_CASE(TTV, MT, PERV, RANKV, GRPV) L1_BWD_CASE6(TTV, MT, PERV, RANKV, GRPV, false)
+	if (p.wide && p.branch_free) {
+		// bwd_plan() sets branch_free only for 64-token tiles with four staged values per thread
+		if (p.rank && p.group > 1) L1_BWD_CASE6(64, 512, 4, true, true, true);
+		else if (p.rank) L1_BWD_CASE6(64, 512, 4, true, false, true);
+		else if (p.group > 1) L1_BWD_CASE6(64, 512, 4, false, true, true);
+		else L1_BWD_CASE6(64, 512, 4, false, false, true);
+	} else if (p.wide && p.group > 1) {
+		// bwd_plan() groups tiles only for these instantiations
+		if (p.rank) L1_BWD_CASE(64, 512, 4, true, true);
+		else if (p.per <= 4) L1_BWD_CASE(64, 512, 4, false, true);
+		else L1_BWD_CASE(64, 512, 8, false, true);
+	} else if (p.wide && p.rank) {
 		switch (p.tt_rows) {
 		case 64:
-			if (p.per <= 4) L1_BWD_CASE(64, 512, 4, true);
-			else L1_BWD_CASE(64, 512, 8, true);
+			if (p.per <= 4) L1_BWD_CASE(64, 512, 4, true, false);
+			else L1_BWD_CASE(64, 512, 8, true, false);
 			break;
-		case 72: L1_BWD_CASE(72, 512, 8, true); break;
-		default: L1_BWD_CASE(80, 512, 8, true); break;
+		case 72: L1_BWD_CASE(72, 512, 8, true, false); break;
+		default: L1_BWD_CASE(80, 512, 8, true, false); break;
 		}
 	} else if (p.wide) {
 		switch (p.tt_rows) {
 		case 64:
-			if (p.per <= 4) L1_BWD_CASE(64, 512, 4, false);
-			else L1_BWD_CASE(64, 512, 8, false);
+			if (p.per <= 4) L1_BWD_CASE(64, 512, 4, false, false);
+			else L1_BWD_CASE(64, 512, 8, false, false);
 			break;
-		case 72: L1_BWD_CASE(72, 512, 8, false); break;
-		case 80: L1_BWD_CASE(80, 512, 8, false); break;
-		default: L1_BWD_CASE(88, 512, 8, false); break;
+		case 72: L1_BWD_CASE(72, 512, 8, false, false); break;
+		case 80: L1_BWD_CASE(80, 512, 8, false, false); break;
+		default: L1_BWD_CASE(88, 512, 8, false, false); break;
 		}
 	} else {
-		if (p.per <= 1) L1_BWD_CASE(32, 1024, 1, false);
-		else if (p.per <= 2) L1_BWD_CASE(32, 1024, 2, false);
-		else if (p.per <= 4) L1_BWD_CASE(32, 1024, 4, false);
-		else if (p.per <= 8) L1_BWD_CASE(32, 1024, 8, false);
-		else L1_BWD_CASE(32, 1024, 16, false);
+		if (p.per <= 1) L1_BWD_CASE(32, 1024, 1, false, false);
+		else if (p.per <= 2) L1_BWD_CASE(32, 1024, 2, false, false);
+		else if (p.per <= 4) L1_BWD_CASE(32, 1024, 4, false, false);
+		else if (p.per <= 8) L1_BWD_CASE(32, 1024, 8, false, false);
+		else L1_BWD_CASE(32, 1024, 16, false, false);
 	}
 #undef L1_BWD_CASE
+#undef L1_BWD_CASE6
 }
 
 }  // namespace
@@ -821,7 +913,7 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 	BwdPlan p = bwd_plan(B, T, H, W);
 	if (!p.fast || p.per_batch_bytes == 0) return 0;
 	// enough batches per launch to put >= 1024 workgroups in flight, never more than B
-	int64_t nb = l1_cdiv(1024, (int64_t)p.n_tt * p.n_cc);
+	int64_t nb = l1_cdiv(1024, (int64_t)p.n_groups * p.n_cc);
 	if (nb > B) nb = B;
 	return p.per_batch_bytes * (size_t)nb;
 }
@@ -847,7 +939,7 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 	if (!workspace || workspace_bytes < p.per_batch_bytes) return L1ATTN_ERR_WORKSPACE;
 	int64_t nb_max = (int64_t)(workspace_bytes / p.per_batch_bytes);
 	if (nb_max > B) nb_max = B;
-	// workspace: [n_tt][nb_max][T][HW] dk partials, then (rank path) rq and rk [nb_max][T][HW] each, the
+	// workspace: [n_groups][nb_max][T][HW] dk partials, then (rank path) rq and rk [nb_max][T][HW] each, the
 	// column sums per dst tile [n_tt][nb_max][T][H] and their total [nb_max][T][H]
 	float* dkp = (float*)workspace;
 	float* rq = dkp + (size_t)nb_max * (p.partial_bytes / sizeof(float));
@@ -856,7 +948,7 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 	float* cs = csp + (size_t)p.n_tt * nb_max * T * H;
 	for (int64_t b0 = 0; b0 < B; b0 += nb_max) {
 		const int64_t nb = std::min<int64_t>(nb_max, B - b0);
-		dim3 grid(p.n_tt, p.n_cc, (unsigned)nb);
+		dim3 grid(p.n_groups, p.n_cc, (unsigned)nb);
 		const float* qa = q + b0 * T * HW;
 		const float* ka = k + b0 * T * HW;
 		if (p.rank) {
@@ -880,7 +972,7 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 		const dim3 rgrid((unsigned)l1_cdiv(ne, vec ? 1024 : 256));
 #define L1_REDUCE_CASE(VECV, RANKV)                                                                             \
 	hipLaunchKernelGGL((dense_bwd_reduce_dk<VECV, RANKV>), rgrid, dim3(256), 0, st, dkp, dk + b0 * T * HW, ne,    \
-	                   p.n_tt, cs, (int)HW, (int)W, (int)H, scale)
+	                   p.n_groups, cs, (int)HW, (int)W, (int)H, scale)
 		if (vec && p.rank) L1_REDUCE_CASE(true, true);
 		else if (vec) L1_REDUCE_CASE(true, false);
 		else if (p.rank) L1_REDUCE_CASE(false, true);

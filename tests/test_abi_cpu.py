@@ -52,8 +52,9 @@ def test_host_side_argument_logic(lib):
     assert lib.l1attn_dense_bwd_workspace_bytes(2, 32, 4, 32) == 0
     assert lib.l1attn_dense_bwd_workspace_bytes(2, 3, 16, 7) == 0
     # headline config: 64 dst tiles (64 tokens each) x 8 batches x T x H*W floats
-    # per batch: 64 dst tiles of dk partials [T][HW], the two rank arrays [T][HW], 64 + 1 column-sum arrays [T][H]
-    assert lib.l1attn_dense_bwd_workspace_bytes(8, 4096, 16, 64) == 8 * 4 * ((64 + 2) * 4096 * 1024 + 65 * 4096 * 16)
+    # per batch: 16 dk partials [T][HW] (64 dst tiles, four per workgroup), the two rank arrays [T][HW],
+    # 64 + 1 column-sum arrays [T][H]
+    assert lib.l1attn_dense_bwd_workspace_bytes(8, 4096, 16, 64) == 8 * 4 * ((16 + 2) * 4096 * 1024 + 65 * 4096 * 16)
     lib.l1attn_dense_fwd_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, vp]
     assert lib.l1attn_dense_fwd_f32(None, None, None, 1, 4, 2, 8, None) == -1      # null pointers
     assert lib.l1attn_dense_fwd_f32(None, None, None, 0, 4, 2, 8, None) == 0       # empty batch: nothing to do
