@@ -28,9 +28,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 # HBM bytes per dense-backward launch (B=8,T=4096,H=16,W=64) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/dense_B8_T4096_H16_W64_pmc_*.txt), scaled by what three 1 GiB device copies read on the same
-# counters (profiles/copy_1GiB_pmc_*.txt: FETCH_SIZE 0.5 per KiB -> x2.0, WRITE_SIZE 1.0 per KiB -> x1.0):
-# main kernel 5291015*2 + 8519680 KiB, dk reduce 4194591*2 + 131072 KiB.
-DENSE_BWD_TRAFFIC_BYTES = (5291015 * 2 + 8519680 + 4194591 * 2 + 131072) * 1024
+# counters (profiles/copy_1GiB_pmc_*.txt: FETCH_SIZE 0.5 per KiB -> x2.0, WRITE_SIZE 1.0 per KiB -> x1.0).
+# KiB per kernel, fetch / write: column ranks 151462 / 262144, main kernel 10975312 / 8650753,
+# column-sum reduce 65548 / 2048, dk reduce 1050657 / 131072.
+DENSE_BWD_TRAFFIC_BYTES = ((151462 + 10975312 + 65548 + 1050657) * 2 + 262144 + 8650753 + 2048 + 131072) * 1024
 
 
 def log(*a):
@@ -252,14 +253,16 @@ def main():
     log(json.dumps(d))
     N = d["pair_elements"]
     roof = {
-        "bound": "valu", "kernel": "dense_bwd_f32_fast (+ dense_bwd_reduce_dk, one backward launch)",
+        "bound": "valu", "kernel": "dense_bwd_f32_fast (+ dense_column_ranks, dense_bwd_reduce_colsum, dense_bwd_reduce_dk: one backward launch)",
         "achieved": d["bwd_tops"], "peak": P_VALU_TOPS, "unit": "TFLOP/s",
         "frac": d["bwd_tops"] / P_VALU_TOPS,
         "traffic": DENSE_BWD_TRAFFIC_BYTES,
         "flops_per_launch": 4 * N, "avg_launch_ms": d["bwd_ms"],
         "note": "algorithmic ops (4 per pair-element) over the HIP-event time of the backward launch; "
                 "peak = nominal fp32 VALU issue rate (one wave64 instruction per SIMD every 2 cycles at "
-                "2.4 GHz); traffic = HBM bytes of the launch against 8.5 GiB algorithmic (dA once + q,k,dq,dk)",
+                "2.4 GHz); traffic = HBM bytes of the launch against 8.5 GiB algorithmic (dA once + q,k,dq,dk): "
+                "the rest is the dk partials (written and re-read by the four dst tiles of a workgroup, read by "
+                "the reduction) and dA lines fetched by both column halves",
     }
     out = {
         "metric": "dense fwd+bwd GOP/s & % fp32 VALU peak; sparse fwd+bwd edges/s & HBM GB/s",
