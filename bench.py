@@ -165,6 +165,29 @@ def sparse_configs(skip_cpu):
     return res
 
 
+def valu_probe():
+    """What ordinary (non-packed) fp32 VALU code sustains on this GPU: the library's register-only probe on
+    256 workgroups of 8 waves (two waves per SIMD on every CU), HIP events on the current stream."""
+    import torch
+    import _l1attn_hip as drv
+    L = drv.lib()
+    blocks, iters = 256, 4000
+    out = torch.empty(blocks * 512, dtype=torch.float32, device="cuda:0")
+    st = drv.stream_of(out)
+    assert L.l1attn_probe_valu(drv.ptr(out), blocks, 100, st) == 0
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    assert L.l1attn_probe_valu(drv.ptr(out), blocks, iters, st) == 0
+    ev[1].record()
+    torch.cuda.synchronize()
+    ms = ev[0].elapsed_time(ev[1])
+    lane_ops = blocks * 8 * iters * 64 * 64
+    tops = lane_ops / (ms * 1e-3) / 1e12
+    return {"kernel": "probe_valu_loop (independent v_fmac_f32, registers only, 2 waves per SIMD)",
+            "lane_tops": tops, "frac_of_nominal_peak": tops / P_VALU_TOPS, "ms": ms}
+
+
 def cpu_baseline():
     """The reference's own CPU extension (oracle/_ref, fp64, one thread, scalar) when it was built and
     carried here, else the C restatement (oracle/liboracle.so, fp64, one thread), on a bounded sample
@@ -274,6 +297,7 @@ def main():
                                "(BASELINE.json configs[2], the headline dense configuration)",
                    "B": 8, "T": 4096, "H": 16, "W": 64},
         "frac_of_fp32_valu_peak": d["frac_of_valu_peak"],
+        "valu_probe": valu_probe(),
         "dense": d,
         "roofline": roof,
     }

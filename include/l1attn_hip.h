@@ -34,6 +34,14 @@ extern "C" {
 /* Library version (major*10000 + minor*100 + patch). */
 int l1attn_version(void);
 
+/*
+ * Measurement aid, no counterpart in the reference: a register-only loop of independent,
+ * non-packed v_fmac_f32 (blocks workgroups of 512 threads, every wave issues iters*64 of them),
+ * to time what the fp32 VALU of the GPU at hand sustains for ordinary code against the nominal
+ * one instruction per SIMD every two cycles.  out: blocks*512 floats.  Asynchronous.
+ */
+int l1attn_probe_valu(float* out, int64_t blocks, int64_t iters, void* stream);
+
 /* ------------------------------------------------------------------------------ dense */
 
 /*

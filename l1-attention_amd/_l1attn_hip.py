@@ -36,6 +36,8 @@ def lib():
                 "libl1attn_hip.so is not built: run `python %s`" % os.path.join(_HERE, "build.py"))
         L = ctypes.CDLL(_LIB_PATH)
         L.l1attn_version.restype = ctypes.c_int
+        L.l1attn_probe_valu.restype = ctypes.c_int
+        L.l1attn_probe_valu.argtypes = [_c_p, _c_i64, _c_i64, _c_p]
         L.l1attn_dense_bwd_workspace_bytes.restype = _c_sz
         L.l1attn_dense_bwd_workspace_bytes.argtypes = [_c_i64] * 4
         for sfx in ("f32", "f64"):

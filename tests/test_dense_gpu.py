@@ -275,3 +275,15 @@ def test_dense_input_checks():
     # the autograd wrapper packs non-contiguous inputs like the reference (cuda/l1attn_cuda.py:11-12)
     a = m.L1AttnFn.apply(qc, qc)
     assert torch.allclose(a.cpu(), cf.dense_attn(qc.cpu().double(), qc.cpu().double()).float(), atol=1e-5)
+
+
+def test_valu_probe_runs():
+    """The measurement aid of the bench: a register-only VALU loop; here only that it runs and writes its output."""
+    import _l1attn_hip as drv
+    L = drv.lib()
+    out = torch.full((4 * 512,), float("nan"), device="cuda")
+    assert L.l1attn_probe_valu(drv.ptr(out), 4, 3, drv.stream_of(out)) == 0
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    assert L.l1attn_probe_valu(None, 4, 3, drv.stream_of(out)) == -1
+    assert L.l1attn_probe_valu(drv.ptr(out), 0, 3, drv.stream_of(out)) == -1
