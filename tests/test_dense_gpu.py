@@ -263,6 +263,76 @@ def test_dense_headline_size_properties():
     assert float((sq + sk).abs().max()) <= 1e-4 * float(sq.abs().max())
 
 
+@pytest.mark.parametrize("W", [16, 32, 33, 64, 65, 96, 97, 128])
+def test_dense_benchmark_grid_widths(W):
+    """The widths of the reference's own timing sweep (benchmark.py:58-60), at two of its sequence lengths."""
+    for T in (16, 128):
+        B, H = 4, 8
+        print("case dense grid", (B, T, H, W), flush=True)
+        q, k, da = _inputs(B, T, H, W, seed=W * 1000 + T)
+        a, dq, dk = _run_gpu(q, k, da)
+        ra = oracle.dense_fwd(q.double(), k.double())
+        rdq, rdk = oracle.dense_bwd(da.double(), q.double(), k.double())
+        assert cf.rel_err(a, ra) <= FWD_TOL
+        assert cf.rel_err(dq, rdq) <= BWD_TOL and cf.rel_err(dk, rdk) <= BWD_TOL
+
+
+def test_dense_layernorm_scaled_inputs():
+    """BASELINE config 3's second input set: unit variance per token and head (LayerNorm over the width)."""
+    print("case dense layernorm inputs", flush=True)
+    B, T, H, W = 2, 320, 16, 64
+    q, k, da = _inputs(B, T, H, W, seed=33)
+    q = torch.nn.functional.layer_norm(q, (W,))
+    k = torch.nn.functional.layer_norm(k, (W,))
+    a, dq, dk = _run_gpu(q, k, da)
+    ra = oracle.dense_fwd(q.double(), k.double())
+    rdq, rdk = oracle.dense_bwd(da.double(), q.double(), k.double())
+    assert cf.rel_err(a, ra) <= FWD_TOL
+    assert cf.rel_err(dq, rdq) <= BWD_TOL and cf.rel_err(dk, rdk) <= BWD_TOL
+
+
+def test_dense_in_a_model_block():
+    """The call pattern of the reference's transformer block (example-setfind/setfind.py:98-138): q from a
+    linear layer, k a gated broadcast view of x, both padded with zero tokens to a multiple of 16, one logit
+    row overwritten with the no-op 0, softmax over src, contraction with v, sum over heads; gradients back
+    to x and the weights.  Yardstick: the same graph in fp64 with the closed form for the logits."""
+    print("case dense model block", flush=True)
+    torch.manual_seed(12)
+    batch, ntok, d_model, n_head = 3, 21, 32, 4
+    m = _mods()
+
+    def block(x, wq, wv, wk, l1a):
+        q = (x @ wq).reshape(batch, ntok, n_head, d_model)
+        v = (x @ wv).reshape(batch, ntok, n_head, d_model)
+        k = x.unsqueeze(2).expand(-1, -1, n_head, -1) * wk.unsqueeze(0).unsqueeze(0)
+        padn = ((ntok + 15) // 16) * 16 - ntok
+        zeros = torch.zeros(batch, padn, n_head, d_model, dtype=x.dtype, device=x.device)
+        a = l1a(torch.cat((q, zeros), 1), torch.cat((k, zeros), 1))
+        a = a[:, :ntok + 1, :ntok, :].clone()
+        a[:, ntok, :, :] = 0.0
+        a = torch.softmax(a, 1)[:, :ntok]
+        return torch.einsum("bsdh,bshw->bdhw", a, v).sum(2)
+
+    def leaves(dtype, device):
+        g = torch.Generator().manual_seed(99)
+        x = torch.randn(batch, ntok, d_model, generator=g)
+        wq = torch.randn(d_model, n_head * d_model, generator=g) / math.sqrt(d_model)
+        wv = torch.randn(d_model, n_head * d_model, generator=g) / math.sqrt(d_model)
+        wk = torch.randn(n_head, d_model, generator=g)
+        return [t.to(dtype).to(device).requires_grad_() for t in (x, wq, wv, wk)]
+
+    got = leaves(torch.float32, "cuda")
+    out = block(*got, m.L1Attn())
+    ref = leaves(torch.float64, "cuda")
+    out_ref = block(*ref, cf.dense_attn)
+    gout = torch.randn(out.shape, generator=torch.Generator().manual_seed(5)).cuda()
+    out.backward(gout)
+    out_ref.backward(gout.double())
+    assert cf.rel_err(out.detach().cpu(), out_ref.detach().cpu()) <= 1e-5
+    for a, b in zip(got, ref):
+        assert cf.rel_err(a.grad.cpu(), b.grad.cpu()) <= BWD_TOL
+
+
 def test_dense_input_checks():
     m = _mods()
     import _l1attn_hip as drv
