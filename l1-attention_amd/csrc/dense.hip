@@ -783,9 +783,12 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.fast = B >= 1 && T >= 16 && HW >= 32 && T <= (1 << 30) && B <= 65535 && HW <= (int64_t)512 * 65535 &&
 	         (BWD_SJ * T + 128) * H < ((int64_t)1 << 31);  // 32-bit staging offsets
 	if (!p.fast) return p;
-	// wide tiles pay off once there are enough dst tokens to give every CU a few workgroups
-	p.wide = T >= 1024 && B * l1_cdiv(HW, 512) * l1_cdiv(T, 88) >= N_CU;
-	const int maxthreads = p.wide ? 512 : 1024;
+	// wide tiles (one workgroup of up to 8 waves per CU) pay off once every CU gets its two waves per SIMD
+	const int64_t wide_threads = std::min<int64_t>(512, l1_cdiv(HW, 64) * 64);
+	p.wide = T >= 1024 && B * l1_cdiv(HW, wide_threads) * l1_cdiv(T, 64) * (wide_threads / 64) >= 8 * N_CU;
+	int maxthreads = p.wide ? 512 : 1024;
+	// narrow tiles: halve the workgroups rather than leave CUs without one
+	if (!p.wide && HW >= 1024 && B * l1_cdiv(HW, 1024) * l1_cdiv(T, 32) < N_CU) maxthreads = 512;
 	p.threads = (int)std::min<int64_t>(maxthreads, l1_cdiv(HW, 64) * 64);
 	p.n_cc = (int)l1_cdiv(HW, p.threads);
 	int64_t hb_exact = 1;  // most heads any column chunk touches

@@ -51,6 +51,7 @@ SHAPES_F32 = [
     (1, 40, 2, 128),    # widest fast width
     (3, 33, 1, 65),     # odd width above 64
     (1, 256, 8, 64),    # benchmark.py grid point
+    (9, 960, 16, 64),   # enough narrow dst tiles for 1024-thread backward workgroups
 ]
 
 
