@@ -56,6 +56,18 @@ int l1attn_dense_fwd_f64(const double* q, const double* k, double* attn,
                          int64_t B, int64_t T, int64_t H, int64_t W, void* stream);
 
 /*
+ * The f32 forward with a workspace.  Widths that are not a multiple of 16 (the reference's timing
+ * sweep uses 33, 65, 97: benchmark.py:60) run the tiled kernels on zero-padded copies of q and k
+ * held in `workspace` (l1attn_dense_fwd_workspace_bytes(), 0 when the shape needs none; 16-byte
+ * aligned); without a workspace they take the generic kernel, as l1attn_dense_fwd_f32 does.
+ * Same results either way up to fp32 summation order.
+ */
+size_t l1attn_dense_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W);
+int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn,
+                            int64_t B, int64_t T, int64_t H, int64_t W,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * dq[b,t,h,w] =  sum_s scale*sign(q[b,t,h,w]-k[b,s,h,w]) * d_attn[b,s,t,h]
  * dk[b,s,h,w] = -sum_t scale*sign(q[b,t,h,w]-k[b,s,h,w]) * d_attn[b,s,t,h],   sign(0) = 0.
  * Replaces l1attn_cuda_drv.backward(d_attn,q,k) -> [dq,dk]  (cuda/l1attn_cuda_drv.cpp:67-104,

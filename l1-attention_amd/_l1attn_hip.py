@@ -38,6 +38,10 @@ def lib():
         L.l1attn_version.restype = ctypes.c_int
         L.l1attn_probe_valu.restype = ctypes.c_int
         L.l1attn_probe_valu.argtypes = [_c_p, _c_i64, _c_i64, _c_p]
+        L.l1attn_dense_fwd_workspace_bytes.restype = _c_sz
+        L.l1attn_dense_fwd_workspace_bytes.argtypes = [_c_i64] * 4
+        L.l1attn_dense_fwd_ws_f32.restype = ctypes.c_int
+        L.l1attn_dense_fwd_ws_f32.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]
         L.l1attn_dense_bwd_workspace_bytes.restype = _c_sz
         L.l1attn_dense_bwd_workspace_bytes.argtypes = [_c_i64] * 4
         for sfx in ("f32", "f64"):
@@ -115,8 +119,14 @@ def dense_forward(q, k):
     B, T, H, W = q.shape
     sfx = sfx_of(q)
     attn = torch.empty((B, T, T, H), dtype=q.dtype, device=q.device)
+    L = lib()
     with torch.cuda.device(q.device):
-        rc = getattr(lib(), "l1attn_dense_fwd_" + sfx)(ptr(q), ptr(k), ptr(attn), B, T, H, W, stream_of(q))
+        ws_bytes = L.l1attn_dense_fwd_workspace_bytes(B, T, H, W) if sfx == "f32" else 0
+        if ws_bytes:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+            rc = L.l1attn_dense_fwd_ws_f32(ptr(q), ptr(k), ptr(attn), B, T, H, W, ptr(ws), ws_bytes, stream_of(q))
+        else:
+            rc = getattr(L, "l1attn_dense_fwd_" + sfx)(ptr(q), ptr(k), ptr(attn), B, T, H, W, stream_of(q))
     check(rc, "l1attn_dense_fwd_" + sfx)
     return [attn]
 

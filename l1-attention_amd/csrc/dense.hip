@@ -674,6 +674,19 @@ __global__ __launch_bounds__(256) void dense_bwd_reduce_dk(const float* __restri
 	}
 }
 
+// qp, kp: rows of q, k copied to width WP and filled up with zeros; n = rows*WP, grid-stride
+__global__ __launch_bounds__(256) void dense_pad_rows(const float* __restrict__ q, const float* __restrict__ k,
+                                                        float* __restrict__ qp, float* __restrict__ kp, int64_t n, int W,
+                                                        int WP)
+{
+	for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+		const int64_t row = i / WP;
+		const int w = (int)(i - row * WP);
+		qp[i] = w < W ? q[row * W + w] : 0.0f;
+		kp[i] = w < W ? k[row * W + w] : 0.0f;
+	}
+}
+
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
@@ -728,8 +741,10 @@ bool fwd_fast_ok(const float* q, const float* k, int64_t B, int64_t T, int64_t H
 	return B * n_hg <= 65535 && T <= (1 << 30) && H <= 65535;
 }
 
+// W: width of the rows the kernels read; W_scale: width the logits are scaled by (smaller when the rows are
+// zero-padded copies)
 int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int64_t Tn, int64_t H, int64_t W,
-                    hipStream_t st)
+                    int64_t W_scale, hipStream_t st)
 {
 	int NH, NTS;
 	fwd_shape(H, Tn, NH, NTS);
@@ -742,7 +757,7 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 	if (s_chunk < 64) s_chunk = 64;
 	int n_sc = (int)l1_cdiv(Tn, s_chunk);
 	if (n_sc > 65535) { s_chunk = l1_cdiv(l1_cdiv(Tn, 65535), FWD_SJ) * FWD_SJ; n_sc = (int)l1_cdiv(Tn, s_chunk); }
-	const float scale = (float)(-1.0 / sqrt((double)W));
+	const float scale = (float)(-1.0 / sqrt((double)W_scale));
 	dim3 grid(n_tt, n_sc, (unsigned)(B * n_hg)), block(64 * NW);
 #define L1_FWD_CASE(KERNEL, WV)                                                                                  \
 	case WV:                                                                                                     \
@@ -887,6 +902,9 @@ void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* d
 
 extern "C" {
 
+int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn, int64_t B, int64_t T, int64_t H, int64_t W,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 int l1attn_dense_fwd_f32(const float* q, const float* k, float* attn, int64_t B, int64_t T, int64_t H, int64_t W,
                          void* stream)
 {
@@ -895,7 +913,45 @@ int l1attn_dense_fwd_f32(const float* q, const float* k, float* attn, int64_t B,
 	if (!q || !k || !attn) return L1ATTN_ERR_ARG;
 	hipStream_t st = (hipStream_t)stream;
 	if (W < 1) return L1ATTN_ERR_ARG;
-	if (fwd_fast_ok(q, k, B, T, H, W)) return launch_fwd_fast(q, k, attn, B, T, H, W, st);
+	return l1attn_dense_fwd_ws_f32(q, k, attn, B, T, H, W, nullptr, 0, stream);
+}
+
+// widths that are not a multiple of 16 run the fast kernels on zero-padded copies of q and k (|0 - 0| adds
+// nothing); the copies cost O(T) against the O(T^2) of the logits
+static int64_t fwd_padded_width(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	if (W % 16 == 0 || W > 128) return 0;
+	const int64_t WP = l1_cdiv(W, 16) * 16;
+	return fwd_fast_ok(nullptr, nullptr, B, T, H, WP) ? WP : 0;
+}
+
+size_t l1attn_dense_fwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	if (!shape_ok(B, T, H, W) || B * T * H * W == 0) return 0;
+	return (size_t)2 * B * T * H * fwd_padded_width(B, T, H, W) * sizeof(float);
+}
+
+int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn, int64_t B, int64_t T, int64_t H, int64_t W,
+                            void* workspace, size_t workspace_bytes, void* stream)
+{
+	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	if (B * T * T * H == 0) return L1ATTN_OK;
+	if (!q || !k || !attn) return L1ATTN_ERR_ARG;
+	hipStream_t st = (hipStream_t)stream;
+	if (W < 1) return L1ATTN_ERR_ARG;
+	if (fwd_fast_ok(q, k, B, T, H, W)) return launch_fwd_fast(q, k, attn, B, T, H, W, W, st);
+	const int64_t WP = fwd_padded_width(B, T, H, W);
+	const int64_t rows = B * T * H;
+	if (WP > 0 && workspace && workspace_bytes >= (size_t)2 * rows * WP * sizeof(float) &&
+	    (((uintptr_t)workspace) & 15) == 0 && 2 * rows * WP < ((int64_t)1 << 40)) {
+		float* qp = (float*)workspace;
+		float* kp = qp + rows * WP;
+		const int64_t n = rows * WP;
+		const dim3 grid((unsigned)std::min<int64_t>(l1_cdiv(n, 256), 1 << 20));
+		hipLaunchKernelGGL(dense_pad_rows, grid, dim3(256), 0, st, q, k, qp, kp, n, (int)W, (int)WP);
+		L1_LAUNCH_CHECK();
+		return launch_fwd_fast(qp, kp, attn, B, T, H, WP, W, st);
+	}
 	return launch_fwd_generic<float>(q, k, attn, B, T, H, W, st);
 }
 

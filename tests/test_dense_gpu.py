@@ -278,6 +278,25 @@ def test_dense_benchmark_grid_widths(W):
         assert cf.rel_err(dq, rdq) <= BWD_TOL and cf.rel_err(dk, rdk) <= BWD_TOL
 
 
+def test_dense_forward_odd_width_with_and_without_workspace():
+    """Widths that are not a multiple of 16: zero-padded copies in a workspace (what the Python wrapper uses)
+    and the workspace-free entry point (generic kernel) both match the oracle."""
+    import _l1attn_hip as drv
+    L = drv.lib()
+    B, T, H, W = 2, 100, 5, 33
+    assert L.l1attn_dense_fwd_workspace_bytes(B, T, H, W) == 2 * B * T * H * 48 * 4
+    assert L.l1attn_dense_fwd_workspace_bytes(B, T, H, 64) == 0
+    assert L.l1attn_dense_fwd_workspace_bytes(B, 8, H, W) == 0      # too few tokens for the tiled kernels
+    q, k, _ = _inputs(B, T, H, W, seed=3)
+    ra = oracle.dense_fwd(q.double(), k.double())
+    qd, kd = q.cuda(), k.cuda()
+    a_ws = drv.dense_forward(qd, kd)[0]
+    a_plain = torch.empty_like(a_ws)
+    assert L.l1attn_dense_fwd_f32(drv.ptr(qd), drv.ptr(kd), drv.ptr(a_plain), B, T, H, W, drv.stream_of(qd)) == 0
+    torch.cuda.synchronize()
+    assert cf.rel_err(a_ws.cpu(), ra) <= FWD_TOL and cf.rel_err(a_plain.cpu(), ra) <= FWD_TOL
+
+
 def test_dense_layernorm_scaled_inputs():
     """BASELINE config 3's second input set: unit variance per token and head (LayerNorm over the width)."""
     print("case dense layernorm inputs", flush=True)
