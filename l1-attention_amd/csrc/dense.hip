@@ -207,8 +207,11 @@ __device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
 template <int W>
 __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restrict__ q, const float* __restrict__ k,
                                                              float* __restrict__ attn, int Tn, int H, int n_hg,
-                                                             int NH, int s_chunk, float scale)
+                                                             int NH, int s_chunk, float scale, int V)
 {
+	// V > 1: q and k rows of width V*W are read as V consecutive heads of width W (the same memory), so
+	// H counts those part-heads, NH (a multiple of V) of them share a workgroup, and the flush adds the V
+	// partial sums of a head.
 	static_assert(W % 32 == 0 && (FWD_SJ % 2) == 0, "chunk stream must keep buffer parity across src blocks");
 	__shared__ float tile[FWD_SJ][FWD_TILE];
 	const int lane = threadIdx.x & 63;
@@ -231,10 +234,12 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
 		}
 	}
-	const int o_tl = threadIdx.x / NH, o_hh = threadIdx.x % NH;
-	const bool o_ok = (tg0 + o_tl < Tn) && (hg * NH + o_hh < H);
-	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (tg0 + o_tl)) * H + hg * NH + o_hh;
-	const int64_t o_pitch = (int64_t)Tn * H;
+	const int NRH = NH / V, H_out = H / V;  // whole heads per workgroup, heads of the output
+	const int o_tl = threadIdx.x / NRH, o_hh = threadIdx.x % NRH;
+	const bool o_ok = (o_tl < NTS * WAVE) && (tg0 + o_tl < Tn) && (hg * NRH + o_hh < H_out);
+	float* const o_base = attn + (((int64_t)b * Tn) * Tn + (tg0 + o_tl)) * H_out + hg * NRH + o_hh;
+	const int64_t o_pitch = (int64_t)Tn * H_out;
+	const int o_lds = o_tl * PH + o_hh * V;
 
 	constexpr int CPR = W / 32;          // chunks per k row
 	constexpr int NCH = FWD_SJ * CPR;    // chunks per src block
@@ -284,7 +289,11 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
 			const int s = s0 + j;
-			if (o_ok && s < s_end) __builtin_nontemporal_store(tile[j][o_tl * PH + o_hh], &o_base[s * o_pitch]);
+			if (o_ok && s < s_end) {
+				float r = tile[j][o_lds];
+				for (int v = 1; v < V; v++) r += tile[j][o_lds + v];
+				__builtin_nontemporal_store(r, &o_base[s * o_pitch]);
+			}
 		}
 		lds_barrier();
 	}
@@ -735,6 +744,7 @@ bool fwd_fast_ok(const float* q, const float* k, int64_t B, int64_t T, int64_t H
 {
 	if (W < 16 || W > 128 || (W % 16) != 0 || T < 32) return false;
 	if ((((uintptr_t)q) | ((uintptr_t)k)) & 15) return false;
+	if (W == 128) H *= 2;  // run as half-heads, see launch_fwd_fast()
 	int NH, NTS;
 	fwd_shape(H, T, NH, NTS);
 	const int64_t n_hg = l1_cdiv(H, NH);
@@ -746,6 +756,11 @@ bool fwd_fast_ok(const float* q, const float* k, int64_t B, int64_t T, int64_t H
 int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int64_t Tn, int64_t H, int64_t W,
                     int64_t W_scale, hipStream_t st)
 {
+	// width 128 runs the pipelined width-64 kernel on half-heads (128 q registers per lane do not leave room
+	// for four waves per SIMD)
+	const int V = W == 128 ? 2 : 1;
+	H *= V;
+	W /= V;
 	int NH, NTS;
 	fwd_shape(H, Tn, NH, NTS);
 	const int NW = NH * NTS;
@@ -764,14 +779,20 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 		hipLaunchKernelGGL(KERNEL<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, NH, (int)s_chunk,    \
 		                   scale);                                                                               \
 		break
+#define L1_FWD_PIPE_CASE(WV)                                                                                     \
+	case WV:                                                                                                     \
+		hipLaunchKernelGGL(dense_fwd_f32_pipe<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, NH,      \
+		                   (int)s_chunk, scale, V);                                                              \
+		break
 	switch (W) {
-		L1_FWD_CASE(dense_fwd_f32_fast, 16); L1_FWD_CASE(dense_fwd_f32_pipe, 32);
-		L1_FWD_CASE(dense_fwd_f32_fast, 48); L1_FWD_CASE(dense_fwd_f32_pipe, 64);
+		L1_FWD_CASE(dense_fwd_f32_fast, 16); L1_FWD_PIPE_CASE(32);
+		L1_FWD_CASE(dense_fwd_f32_fast, 48); L1_FWD_PIPE_CASE(64);
 		L1_FWD_CASE(dense_fwd_f32_fast, 80); L1_FWD_CASE(dense_fwd_f32_fast, 96);
-		L1_FWD_CASE(dense_fwd_f32_fast, 112); L1_FWD_CASE(dense_fwd_f32_fast, 128);
+		L1_FWD_CASE(dense_fwd_f32_fast, 112);
 	default: return L1ATTN_ERR_ARG;
 	}
 #undef L1_FWD_CASE
+#undef L1_FWD_PIPE_CASE
 	L1_LAUNCH_CHECK();
 	return L1ATTN_OK;
 }
@@ -921,7 +942,8 @@ int l1attn_dense_fwd_f32(const float* q, const float* k, float* attn, int64_t B,
 static int64_t fwd_padded_width(int64_t B, int64_t T, int64_t H, int64_t W)
 {
 	if (W % 16 == 0 || W > 128) return 0;
-	const int64_t WP = l1_cdiv(W, 16) * 16;
+	// above 96 the pipelined half-head kernel of width 128 beats the width-112 kernel
+	const int64_t WP = W > 96 ? 128 : l1_cdiv(W, 16) * 16;
 	return fwd_fast_ok(nullptr, nullptr, B, T, H, WP) ? WP : 0;
 }
 
