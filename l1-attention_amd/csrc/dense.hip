@@ -68,6 +68,36 @@ __global__ __launch_bounds__(256) void dense_fwd_generic(const T* __restrict__ q
 	}
 }
 
+// Short sequences (fewer tokens than the tiled kernels need): one workgroup per (b,h) keeps the T q rows and
+// T k rows of the head in LDS (row pitch W+1, so that lanes with consecutive dst tokens hit different banks)
+// and every thread computes whole logits.
+template <typename T>
+__global__ __launch_bounds__(256) void dense_fwd_small(const T* __restrict__ q, const T* __restrict__ k,
+                                                         T* __restrict__ attn, int Tn, int H, int W, T scale)
+{
+	extern __shared__ unsigned char small_lds[];
+	T* const qs = reinterpret_cast<T*>(small_lds);
+	const int WP = W + 1;
+	T* const ks = qs + Tn * WP;
+	const int64_t b = blockIdx.x / (unsigned)H;
+	const int h = (int)(blockIdx.x % (unsigned)H);
+	for (int i = threadIdx.x; i < Tn * W; i += 256) {
+		const int t = i / W, w = i - t * W;
+		const int64_t off = ((b * Tn + t) * H + h) * (int64_t)W + w;
+		qs[t * WP + w] = q[off];
+		ks[t * WP + w] = k[off];
+	}
+	__syncthreads();
+	for (int o = threadIdx.x; o < Tn * Tn; o += 256) {
+		const int s = o / Tn, t = o - s * Tn;
+		const T* qp = qs + t * WP;
+		const T* kp = ks + s * WP;
+		T f = 0;
+		for (int w = 0; w < W; w++) f += abs_t(qp[w] - kp[w]);
+		attn[((b * Tn + s) * Tn + t) * H + h] = f * scale;
+	}
+}
+
 // one thread per dq element, src tokens summed in ascending order
 template <typename T>
 __global__ __launch_bounds__(256) void dense_bwd_generic_dq(const T* __restrict__ dA, const T* __restrict__ q,
@@ -709,6 +739,13 @@ template <typename T>
 int launch_fwd_generic(const T* q, const T* k, T* attn, int64_t B, int64_t Tn, int64_t H, int64_t W, hipStream_t st)
 {
 	const T scale = (T)(-1.0 / sqrt((double)W));
+	const size_t small_bytes = (size_t)2 * Tn * (W + 1) * sizeof(T);
+	if (Tn <= 64 && small_bytes <= 48 * 1024 && B * H < ((int64_t)1 << 31)) {
+		hipLaunchKernelGGL(dense_fwd_small<T>, dim3((unsigned)(B * H)), dim3(256), small_bytes, st, q, k, attn, (int)Tn,
+		                   (int)H, (int)W, scale);
+		L1_LAUNCH_CHECK();
+		return L1ATTN_OK;
+	}
 	dim3 grid((unsigned)l1_cdiv(Tn * H, 256), (unsigned)std::min<int64_t>(B * Tn, 65535), 1);
 	hipLaunchKernelGGL(dense_fwd_generic<T>, grid, dim3(256), 0, st, q, k, attn, B, Tn, H, W, scale);
 	L1_LAUNCH_CHECK();

@@ -69,7 +69,7 @@ def test_dense_f32_vs_oracle(shape):
     assert cf.rel_err(dk, rdk) <= BWD_TOL
 
 
-@pytest.mark.parametrize("shape", [(2, 64, 4, 32), (1, 16, 8, 64), (2, 5, 3, 7)])
+@pytest.mark.parametrize("shape", [(2, 64, 4, 32), (1, 16, 8, 64), (2, 5, 3, 7), (1, 100, 3, 33)])
 def test_dense_f64_vs_oracle(shape):
     B, T, H, W = shape
     print("case dense f64", shape, flush=True)
