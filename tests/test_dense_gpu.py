@@ -203,6 +203,33 @@ def test_dense_backward_long_sequences_vs_oracle(shape, tag):
     assert tie_dq <= 1e-5 and tie_dk <= 1e-5
 
 
+def test_dense_backward_small_workspace_loops_over_batches():
+    """A workspace of one batch's share makes the library process the batches in several launches; same bits
+    as with the full workspace (rank path, so the rank arrays and column sums are offset per launch too)."""
+    import _l1attn_hip as drv
+    L = drv.lib()
+    B, T, H, W = 3, 2048, 32, 64
+    print("case dense small workspace", (B, T, H, W), flush=True)
+    g = torch.Generator(device="cuda").manual_seed(8)
+    q = torch.randn(B, T, H, W, generator=g, device="cuda")
+    k = torch.randn(B, T, H, W, generator=g, device="cuda")
+    da = torch.randn(B, T, T, H, generator=g, device="cuda")
+    dq_full, dk_full = drv.dense_backward(da, q, k)
+    full = L.l1attn_dense_bwd_workspace_bytes(B, T, H, W)
+    assert full % B == 0
+    one = full // B
+    ws = torch.empty(one + 100, dtype=torch.uint8, device="cuda")   # room for exactly one batch
+    dq, dk = torch.empty_like(q), torch.empty_like(k)
+    rc = L.l1attn_dense_bwd_f32(drv.ptr(da), drv.ptr(q), drv.ptr(k), drv.ptr(dq), drv.ptr(dk), B, T, H, W,
+                                drv.ptr(ws), one + 100, drv.stream_of(q))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dq, dq_full) and torch.equal(dk, dk_full)
+    rc = L.l1attn_dense_bwd_f32(drv.ptr(da), drv.ptr(q), drv.ptr(k), drv.ptr(dq), drv.ptr(dk), B, T, H, W,
+                                drv.ptr(ws), one - 4, drv.stream_of(q))
+    assert rc == -2   # smaller than one batch's share
+
+
 def test_dense_column_ranks():
     """First stage of the long-sequence backward: the rank maps keep order and ties of every column."""
     import ctypes
