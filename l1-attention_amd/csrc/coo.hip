@@ -31,6 +31,32 @@ constexpr int RS_DIGITS = 1 << RS_BITS;
 // stats words written by the extract kernels
 enum { ST_MAXKEY = 0, ST_BAD = 1, ST_MAXDEG_DST = 2, ST_MAXDEG_SRC = 3, ST_NLONG_DST = 4, ST_NLONG_SRC = 5, ST_WORDS = 8 };
 
+// maximum over the wave's 64 lanes (every lane must call it), returned in all lanes
+__device__ __forceinline__ int wave_max(int v)
+{
+#pragma unroll
+	for (int off = 32; off >= 1; off >>= 1) {
+		const int o = __shfl_xor(v, off, 64);
+		v = o > v ? o : v;
+	}
+	return v;
+}
+
+// maximum over the workgroup (256 threads, every thread must call it), valid in thread 0
+__device__ __forceinline__ int block_max_256(int v)
+{
+	__shared__ int wm[4];
+	v = wave_max(v);
+	if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = v;
+	__syncthreads();
+	const int a = wm[0] > wm[1] ? wm[0] : wm[1], b = wm[2] > wm[3] ? wm[2] : wm[3];
+	return a > b ? a : b;
+}
+
+constexpr int ROWS_PER_THREAD = 8;  // rows per thread of the row-parallel kernels below
+
+// Same-address atomics are served one at a time by the L2 (about 10 ns each, whatever the wave coalesces),
+// so the row-parallel kernels reduce over a workgroup of 2048 rows first and issue one atomic.
 template <typename IdxT>
 __global__ __launch_bounds__(256) void coo_extract(const IdxT* __restrict__ co, int64_t stride, int64_t E,
                                                      int* __restrict__ dst32, int* __restrict__ src32,
@@ -38,23 +64,33 @@ __global__ __launch_bounds__(256) void coo_extract(const IdxT* __restrict__ co, 
 {
 	// n_tok < 0: any non-negative int32 index is valid (expandCoo); otherwise indices must be < n_tok
 	// and invalid rows get the sentinel key n_tok in both columns (they sort last and are dropped).
-	const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-	if (i >= E) return;
-	const long long d = (long long)co[i * stride], s = (long long)co[i * stride + 1];
-	const long long hi = n_tok < 0 ? 2147483647LL : (long long)n_tok - 1;
-	const bool bad = d < 0 || s < 0 || d > hi || s > hi;
-	int di = (int)d, si = (int)s;
-	if (bad) {
-		atomicOr(&stats[ST_BAD], 1);
-		di = si = n_tok < 0 ? 0 : (int)n_tok;
+	int key_max = 0;
+	bool any_bad = false;
+#pragma unroll
+	for (int it = 0; it < ROWS_PER_THREAD; it++) {
+		const int64_t i = ((int64_t)blockIdx.x * ROWS_PER_THREAD + it) * 256 + threadIdx.x;
+		if (i < E) {
+			const long long d = (long long)co[i * stride], s = (long long)co[i * stride + 1];
+			const long long hi = n_tok < 0 ? 2147483647LL : (long long)n_tok - 1;
+			const bool bad = d < 0 || s < 0 || d > hi || s > hi;
+			int di = (int)d, si = (int)s;
+			if (bad) {
+				any_bad = true;
+				di = si = n_tok < 0 ? 0 : (int)n_tok;
+			}
+			dst32[i] = di;
+			src32[i] = si;
+			const int m = di > si ? di : si;
+			key_max = m > key_max ? m : key_max;
+			if (coo_out) {
+				coo_out[i * 4 + 0] = di;
+				coo_out[i * 4 + 1] = si;
+			}
+		}
 	}
-	dst32[i] = di;
-	src32[i] = si;
-	atomicMax(&stats[ST_MAXKEY], di > si ? di : si);
-	if (coo_out) {
-		coo_out[i * 4 + 0] = di;
-		coo_out[i * 4 + 1] = si;
-	}
+	if (any_bad) atomicOr(&stats[ST_BAD], 1);
+	key_max = block_max_256(key_max);
+	if (threadIdx.x == 0) atomicMax(&stats[ST_MAXKEY], key_max);
 }
 
 __global__ __launch_bounds__(RS_THREADS) void radix_hist(const int* __restrict__ keys, int64_t E, int shift,
@@ -73,27 +109,59 @@ __global__ __launch_bounds__(RS_THREADS) void radix_hist(const int* __restrict__
 	hist[(int64_t)threadIdx.x * nblk + blockIdx.x] = h[threadIdx.x];
 }
 
-// exclusive prefix sum of n ints in place, one workgroup of 1024 threads
+// Exclusive prefix sum of n ints in place, one workgroup of 1024 threads.  The array is walked in chunks of
+// 8192: a thread takes eight consecutive elements (two 16-byte loads, so a wave reads 2 KiB contiguously),
+// the waves combine their totals with shuffles and one pass through LDS, and the running total carries over.
+// The 16-byte accesses are used when a is 16-byte aligned.
 __global__ __launch_bounds__(1024) void scan_exclusive(int* __restrict__ a, int64_t n)
 {
-	__shared__ int part[1024];
-	const int64_t per = (n + 1023) / 1024;
-	const int64_t lo = (int64_t)threadIdx.x * per, hi = lo + per < n ? lo + per : n;
-	int sum = 0;
-	for (int64_t i = lo; i < hi; i++) sum += a[i];
-	part[threadIdx.x] = sum;
-	__syncthreads();
-	for (int off = 1; off < 1024; off <<= 1) {
-		int v = threadIdx.x >= (unsigned)off ? part[threadIdx.x - off] : 0;
+	__shared__ int wave_total[16];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const bool vec = (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+	int carry = 0;
+	for (int64_t base = 0; base < n; base += 8192) {
+		const int64_t i0 = base + (int64_t)threadIdx.x * 8;
+		int v[8];
+		if (vec && i0 + 8 <= n) {
+			const int4 x = *reinterpret_cast<const int4*>(a + i0), y = *reinterpret_cast<const int4*>(a + i0 + 4);
+			v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w; v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+		} else {
+#pragma unroll
+			for (int j = 0; j < 8; j++) v[j] = i0 + j < n ? a[i0 + j] : 0;
+		}
+		int total = 0;
+#pragma unroll
+		for (int j = 0; j < 8; j++) {  // v[j] becomes the sum of the thread's elements before j
+			const int t = v[j];
+			v[j] = total;
+			total += t;
+		}
+		int incl = total;  // inclusive scan of the thread totals over the wave
+#pragma unroll
+		for (int off = 1; off < 64; off <<= 1) {
+			const int up = __shfl_up(incl, off, 64);
+			if (lane >= off) incl += up;
+		}
+		if (lane == 63) wave_total[wave] = incl;
 		__syncthreads();
-		part[threadIdx.x] += v;
-		__syncthreads();
-	}
-	int run = part[threadIdx.x] - sum;
-	for (int64_t i = lo; i < hi; i++) {
-		const int v = a[i];
-		a[i] = run;
-		run += v;
+		int before = carry, all = 0;
+#pragma unroll
+		for (int w = 0; w < 16; w++) {
+			const int t = wave_total[w];
+			if (w < wave) before += t;
+			all += t;
+		}
+		const int mine = before + incl - total;  // everything before this thread's first element
+		if (vec && i0 + 8 <= n) {
+			*reinterpret_cast<int4*>(a + i0) = make_int4(mine + v[0], mine + v[1], mine + v[2], mine + v[3]);
+			*reinterpret_cast<int4*>(a + i0 + 4) = make_int4(mine + v[4], mine + v[5], mine + v[6], mine + v[7]);
+		} else {
+#pragma unroll
+			for (int j = 0; j < 8; j++)
+				if (i0 + j < n) a[i0 + j] = mine + v[j];
+		}
+		carry += all;
+		__syncthreads();  // wave_total is rewritten by the next chunk
 	}
 }
 
@@ -165,11 +233,18 @@ __global__ __launch_bounds__(256) void ranks_from_sorted(const int* __restrict__
                                                            int* __restrict__ out, int out_stride, int out_col,
                                                            int* __restrict__ maxdeg)
 {
-	const int p = blockIdx.x * 256 + threadIdx.x;
-	if (p >= E) return;
-	const int r = p - lower_bound(keys_sorted, E, keys_sorted[p]);
-	out[(int64_t)rows_sorted[p] * out_stride + out_col] = r;
-	atomicMax(maxdeg, r + 1);
+	int deg = 0;
+#pragma unroll
+	for (int it = 0; it < ROWS_PER_THREAD; it++) {
+		const int64_t p = ((int64_t)blockIdx.x * ROWS_PER_THREAD + it) * 256 + threadIdx.x;
+		if (p < E) {
+			const int r = (int)p - lower_bound(keys_sorted, E, keys_sorted[p]);
+			out[(int64_t)rows_sorted[p] * out_stride + out_col] = r;
+			deg = r + 1 > deg ? r + 1 : deg;
+		}
+	}
+	deg = block_max_256(deg);
+	if (threadIdx.x == 0) atomicMax(maxdeg, deg);
 }
 
 __global__ __launch_bounds__(256) void segment_ptrs(const int* __restrict__ keys_sorted, int E, int n_ptr,
@@ -210,10 +285,10 @@ __global__ __launch_bounds__(256) void max_segment(const int* __restrict__ ptr, 
                                                      int* __restrict__ long_list, int* __restrict__ n_long)
 {
 	const int key = blockIdx.x * 256 + threadIdx.x;
-	if (key >= n_keys) return;
-	const int deg = ptr[key + 1] - ptr[key];
-	atomicMax(out, deg);
+	const int deg = key < n_keys ? ptr[key + 1] - ptr[key] : 0;
 	if (deg > PLAN_LONG_SEGMENT) long_list[atomicAdd(n_long, 1)] = key;
+	const int wmax = wave_max(deg);
+	if ((threadIdx.x & 63) == 0) atomicMax(out, wmax);
 }
 
 __global__ void fill_words(int* __restrict__ a, int n, int v)
@@ -323,14 +398,15 @@ int l1attn_expand_coo(const void* co, int co_bits, int64_t co_stride, int64_t E,
 	int* src32 = (int*)p; p += l1_align_up((size_t)E * 4, 256);
 	const SortBufs sb = carve_sort(p, E);
 	const unsigned g256 = (unsigned)l1_cdiv(E, 256);
+	const unsigned g2048 = (unsigned)l1_cdiv(E, 256 * ROWS_PER_THREAD);
 
 	hipLaunchKernelGGL(fill_words, dim3(1), dim3(64), 0, st, stats, ST_WORDS, 0);
 	L1_LAUNCH_CHECK();
 	if (co_bits == 64)
-		hipLaunchKernelGGL(coo_extract<long long>, dim3(g256), dim3(256), 0, st, (const long long*)co, co_stride, E,
+		hipLaunchKernelGGL(coo_extract<long long>, dim3(g2048), dim3(256), 0, st, (const long long*)co, co_stride, E,
 		                   dst32, src32, coo, (int64_t)-1, stats);
 	else
-		hipLaunchKernelGGL(coo_extract<int>, dim3(g256), dim3(256), 0, st, (const int*)co, co_stride, E, dst32, src32,
+		hipLaunchKernelGGL(coo_extract<int>, dim3(g2048), dim3(256), 0, st, (const int*)co, co_stride, E, dst32, src32,
 		                   coo, (int64_t)-1, stats);
 	L1_LAUNCH_CHECK();
 	int h_stats[ST_WORDS];
@@ -342,12 +418,12 @@ int l1attn_expand_coo(const void* co, int co_bits, int64_t co_stride, int64_t E,
 	const int *ks, *rs;
 	int rc = sort_rows_by_key(dst32, E, bits, sb, st, &ks, &rs);
 	if (rc) return rc;
-	hipLaunchKernelGGL(ranks_from_sorted, dim3(g256), dim3(256), 0, st, ks, rs, (int)E, coo, 4, 2,
+	hipLaunchKernelGGL(ranks_from_sorted, dim3(g2048), dim3(256), 0, st, ks, rs, (int)E, coo, 4, 2,
 	                   stats + ST_MAXDEG_DST);
 	L1_LAUNCH_CHECK();
 	rc = sort_rows_by_key(src32, E, bits, sb, st, &ks, &rs);
 	if (rc) return rc;
-	hipLaunchKernelGGL(ranks_from_sorted, dim3(g256), dim3(256), 0, st, ks, rs, (int)E, coo, 4, 3,
+	hipLaunchKernelGGL(ranks_from_sorted, dim3(g2048), dim3(256), 0, st, ks, rs, (int)E, coo, 4, 3,
 	                   stats + ST_MAXDEG_SRC);
 	L1_LAUNCH_CHECK();
 	L1_HIP_CHECK(hipMemcpyAsync(h_stats, stats, sizeof(h_stats), hipMemcpyDeviceToHost, st));
@@ -403,12 +479,13 @@ int l1attn_sparse_plan_build(const int32_t* coo, int64_t coo_stride, int64_t E, 
 	int* slot_of_row = (int*)p; p += ea;
 	const SortBufs sb = carve_sort(p, E);
 	const unsigned g256 = (unsigned)l1_cdiv(E, 256);
+	const unsigned g2048 = (unsigned)l1_cdiv(E, 256 * ROWS_PER_THREAD);
 	const unsigned gptr = (unsigned)l1_cdiv(T + 2, 256);
 	const int bits = bits_for(T);  // keys 0..T (T = sentinel of invalid rows)
 
 	hipLaunchKernelGGL(fill_words, dim3(1), dim3(64), 0, st, stats, ST_WORDS, 0);
 	L1_LAUNCH_CHECK();
-	hipLaunchKernelGGL(coo_extract<int>, dim3(g256), dim3(256), 0, st, (const int*)coo, coo_stride, E, dst32, src32,
+	hipLaunchKernelGGL(coo_extract<int>, dim3(g2048), dim3(256), 0, st, (const int*)coo, coo_stride, E, dst32, src32,
 	                   (int*)nullptr, T, stats);
 	L1_LAUNCH_CHECK();
 
