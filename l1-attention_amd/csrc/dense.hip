@@ -136,6 +136,7 @@ __global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict_
 // ------------------------------------------------------------------------------------------
 
 constexpr int FWD_SJ = 8;  // src rows finished between two output flushes
+constexpr int FWD_L2_AHEAD = 4;  // src blocks between the L2 prefetch of k rows and their use
 constexpr int FWD_TILE = 1024 + 4 * WAVE;  // floats per staged src row: 64*NW outputs + one pad column per sub-tile (NH >= 4)
 
 // Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.
@@ -286,6 +287,10 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 	sload32(b0l, b0h, kp);
 	__builtin_amdgcn_sched_barrier(0);
 	for (int s0 = s_begin; s0 < s_end; s0 += FWD_SJ) {
+		// Pull the k rows of a later src block into the L2 with one vector load per wave (eight lanes per
+		// row): the scalar loads below then miss the scalar cache but not the L2.  The value is not used;
+		// it is taken before the flush, by which time it has long arrived.
+		const float pf = kb[(int64_t)min(s0 + FWD_L2_AHEAD * FWD_SJ + (lane >> 3), Tn - 1) * krow + (lane & 7) * (W / 8)];
 		float a = 0.0f;
 #pragma unroll
 		for (int c = 0; c < NCH; c++) {
@@ -315,6 +320,7 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 			}
 			if (part == CPR - 1) tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
 		}
+		asm volatile("" ::"v"(pf));
 		lds_barrier();
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
@@ -436,6 +442,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
                                                                    float* __restrict__ csp, int Tn, int H, int W,
                                                                    float scale, int G)
 {
+	static_assert(!FAST || PER == BWD_SJ, "branch-free form: one staged value per thread and src row");
 	constexpr int TTP = TT + 4;  // LDS row pitch: keeps 16-byte alignment for ds_read_b128
 	constexpr int tt_rows = TT;
 	constexpr int NR = (PER + BWD_SJ - 1) / BWD_SJ;  // (head, dst token) slots per thread, >= HB*TT / blockDim.x
@@ -508,7 +515,11 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	// loads of the dA and k values of the step that starts at src token s0
 	auto prefetch = [&](int s0) {
 		const float* const dA_s = dA_b + (int64_t)s0 * Tn * H;  // wave-uniform
-		if (FAST || (full && s0 + BWD_SJ <= Tn)) {
+		if (FAST) {
+			// PER == BWD_SJ and blockDim.x elements per src row: role r is role 0 one src row further on
+#pragma unroll
+			for (int r = 0; r < PER; r++) g_pre[r] = (dA_s + (int64_t)r * Tn * H)[st_off[0]];
+		} else if (full && s0 + BWD_SJ <= Tn) {
 #pragma unroll
 			for (int r = 0; r < PER; r++) g_pre[r] = dA_s[st_off[r]];
 		} else {
@@ -538,7 +549,10 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 
 	for (int s0 = 0; s0 < Tn; s0 += BWD_SJ) {
 		lds_barrier();  // the previous step's LDS reads are done
-		if (full) {
+		if (FAST) {
+#pragma unroll
+			for (int r = 0; r < PER; r++) gl[st_lds[0] + r * HB * TTP] = g_pre[r];
+		} else if (full) {
 #pragma unroll
 			for (int r = 0; r < PER; r++) gl[st_lds[r]] = g_pre[r];
 		} else {
@@ -571,10 +585,13 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			for (int j = 0; j < BWD_SJ; j++) dk_old[j] = (dkp_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
 		}
 		{
-			// all dA values of this step for the lane's head, read one float4 ahead of their use
+			// all dA values of this step for the lane's head, read D float4 ahead of their use
 			const float4* gp0 = reinterpret_cast<const float4*>(gl + hl * TTP);
-			constexpr int NI4 = TT / 4;
-			float4 g_cur = gp0[0];
+			constexpr int NI4 = TT / 4, NBLK = BWD_SJ * NI4, D = FAST ? 2 : 1;
+			auto g_at = [&](int bi) { return gp0[((bi / NI4) * HB * TTP) / 4 + bi % NI4]; };
+			float4 g_ring[D + 1];
+#pragma unroll
+			for (int d = 0; d < D; d++) g_ring[d] = g_at(d);
 			// RANK: the tile values for the sums are read here and added up after the first src row's math,
 			// by which time they have arrived.  Column sums: row = jj*HB + hh of the tile, sixteen lanes per
 			// row (the host checks BWD_SJ*HB*16 <= blockDim.x).  Row sums: this thread's (head, dst token) slots.
@@ -596,12 +613,10 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 				}
 			}
 #pragma unroll
-			for (int j = 0; j < BWD_SJ; j++) {
-#pragma unroll
-				for (int i4 = 0; i4 < NI4; i4++) {
-					float4 g_nxt = g_cur;
-					if (i4 + 1 < NI4) g_nxt = gp0[(j * HB * TTP) / 4 + i4 + 1];
-					else if (j + 1 < BWD_SJ) g_nxt = gp0[((j + 1) * HB * TTP) / 4];
+			for (int bi = 0; bi < NBLK; bi++) {
+				{
+					const int j = bi / NI4, i4 = bi % NI4;
+					if (bi + D < NBLK) g_ring[(bi + D) % (D + 1)] = g_at(bi + D);
 					__builtin_amdgcn_sched_barrier(0);
 					if (RANK && j == 1 && i4 == 0) {
 						// keep the loaded values opaque up to here, or the adds (and the wait for the loads)
@@ -624,9 +639,8 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 						for (int n = 0; n < NR; n++) rs_acc[n] += (rs_v[n][0] + rs_v[n][1]) + (rs_v[n][2] + rs_v[n][3]);
 						__builtin_amdgcn_sched_barrier(0);
 					}
-					if (RANK) pair_step4_rank(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
-					else pair_step4(&qc[i4 * 4], kc[j], g_cur, &dqa[i4 * 4], dka[j]);
-					g_cur = g_nxt;
+					if (RANK) pair_step4_rank(&qc[i4 * 4], kc[j], g_ring[bi % (D + 1)], &dqa[i4 * 4], dka[j]);
+					else pair_step4(&qc[i4 * 4], kc[j], g_ring[bi % (D + 1)], &dqa[i4 * 4], dka[j]);
 				}
 			}
 		}
