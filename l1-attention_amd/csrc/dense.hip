@@ -197,16 +197,21 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 
 	const int s_begin = lb.y * s_chunk;
 	const int s_end = min(Tn, s_begin + s_chunk);
+	const float* const kb = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;  // row 0 of this (b,h), wave-uniform
+	const int64_t krow = (int64_t)H * W;
 	for (int s0 = s_begin; s0 < s_end; s0 += FWD_SJ) {
+		// L2 prefetch of a later src block's k rows, see dense_fwd_f32_pipe
+		const float pf = kb[(int64_t)min(s0 + FWD_L2_AHEAD * FWD_SJ + (lane >> 3), Tn - 1) * krow + (lane & 7) * (W / 8)];
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
 			const int s = min(s0 + j, Tn - 1);
-			const float* kp = k + (((int64_t)b * Tn + s) * H + h) * (int64_t)W;  // wave-uniform -> scalar loads
+			const float* kp = kb + s * krow;  // wave-uniform -> scalar loads
 			float a = 0.0f;
 #pragma unroll
 			for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
 			tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
 		}
+		asm volatile("" ::"v"(pf));
 		lds_barrier();
 #pragma unroll
 		for (int j = 0; j < FWD_SJ; j++) {
@@ -838,7 +843,7 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 	switch (W) {
 		L1_FWD_CASE(dense_fwd_f32_fast, 16); L1_FWD_PIPE_CASE(32);
 		L1_FWD_CASE(dense_fwd_f32_fast, 48); L1_FWD_PIPE_CASE(64);
-		L1_FWD_CASE(dense_fwd_f32_fast, 80); L1_FWD_CASE(dense_fwd_f32_fast, 96);
+		L1_FWD_CASE(dense_fwd_f32_fast, 80); L1_FWD_PIPE_CASE(96);
 		L1_FWD_CASE(dense_fwd_f32_fast, 112);
 	default: return L1ATTN_ERR_ARG;
 	}
