@@ -346,7 +346,25 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 // ------------------------------------------------------------------------------------------
 
 constexpr int BWD_SJ = 4;  // src tokens per staging step
+constexpr int BWD_LDS_BATCH = 4;  // float4 reads of the staged tile issued together in the branch-free form
 constexpr float BWD_PRESCALE = 18446744073709551616.0f;  // 2^64
+
+// Raw buffer access for the branch-free step loop: a uniform base (descriptor in four SGPRs), a per-lane byte
+// offset and a uniform byte offset.  Neither offset costs an instruction per access, where a flat global
+// access takes a 64-bit VALU add for the address and scalar multiplies for the row.
+using buf_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ buf_t make_buf(const void* base)
+{
+	return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);  // raw, no bounds below 4 GiB
+}
+__device__ __forceinline__ float buf_load(buf_t r, unsigned lane_bytes, unsigned uniform_bytes)
+{
+	return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_bytes, (int)uniform_bytes, 0));
+}
+__device__ __forceinline__ void buf_store(float v, buf_t r, unsigned lane_bytes, unsigned uniform_bytes)
+{
+	__builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, (int)lane_bytes, (int)uniform_bytes, 0);
+}
 
 // Sum over each aligned group of 16 lanes (a DPP row); the total lands in the group's last lane.
 // Lanes shifted in from outside the row read as zero.
@@ -518,13 +536,25 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	// branches of the general form cost about 4 % of the kernel).
 	const bool full = FAST || (t0 + tt_rows <= Tn && n_stage == PER * (int)blockDim.x);
 	// loads of the dA and k values of the step that starts at src token s0
+	// FAST: running uniform pointers instead of a multiplication per row: the step being prefetched (dA, k)
+	// and the step being computed (dk partial rows)
+	const float* dA_pf = dA_b;
+	const float* k_pf = k_b;
+	float* dkp_cur = dkp_b;
+	const unsigned row_bytes = HW * 4u, dA_row_bytes = (unsigned)(Tn * H) * 4u, col_bytes = col * 4u;
+	const int64_t dA_step = (int64_t)BWD_SJ * Tn * H, k_step = (int64_t)BWD_SJ * HW;
 	auto prefetch = [&](int s0) {
-		const float* const dA_s = dA_b + (int64_t)s0 * Tn * H;  // wave-uniform
 		if (FAST) {
 			// PER == BWD_SJ and blockDim.x elements per src row: role r is role 0 one src row further on
+			const buf_t rd = make_buf(dA_pf), rk = make_buf(k_pf);
 #pragma unroll
-			for (int r = 0; r < PER; r++) g_pre[r] = (dA_s + (int64_t)r * Tn * H)[st_off[0]];
-		} else if (full && s0 + BWD_SJ <= Tn) {
+			for (int r = 0; r < PER; r++) g_pre[r] = buf_load(rd, st_off[0] * 4u, (unsigned)r * dA_row_bytes);
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) k_pre[j] = buf_load(rk, col_bytes, (unsigned)j * row_bytes);
+			return;
+		}
+		const float* const dA_s = dA_b + (int64_t)s0 * Tn * H;  // wave-uniform
+		if (full && s0 + BWD_SJ <= Tn) {
 #pragma unroll
 			for (int r = 0; r < PER; r++) g_pre[r] = dA_s[st_off[r]];
 		} else {
@@ -535,8 +565,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			}
 		}
 #pragma unroll
-		for (int j = 0; j < BWD_SJ; j++)
-			k_pre[j] = (k_b + (int64_t)(FAST ? s0 + j : min(s0 + j, Tn - 1)) * HW)[col];
+		for (int j = 0; j < BWD_SJ; j++) k_pre[j] = (k_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
 	};
 	// Wait for the prefetched values.  Loads and stores share one counter and may complete out of
 	// order, so a wait for a load while a store is in flight is a wait for everything.  The values
@@ -572,17 +601,22 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			dka[j] = 0.0f;
 		}
 		lds_barrier();
-		// next step's values; FAST: the last step reads the last rows again, and nobody uses them
-		if (FAST) prefetch(min(s0 + BWD_SJ, Tn - BWD_SJ));
-		else if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
+		// next step's values; FAST: the last step reads its own rows again, and nobody uses them
+		if (FAST) {
+			const bool more = s0 + BWD_SJ < Tn;
+			dA_pf += more ? dA_step : 0;
+			k_pf += more ? k_step : 0;
+			prefetch(more ? s0 + BWD_SJ : s0);
+		} else if (s0 + BWD_SJ < Tn) prefetch(s0 + BWD_SJ);
 		// what the earlier tiles of this workgroup left in the partial rows of this step; used after the math
 		float dk_old[BWD_SJ];
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) dk_old[j] = 0.0f;
+		const buf_t rp = make_buf(dkp_cur);
 		if (GROUPED && FAST) {
 #pragma unroll
 			for (int j = 0; j < BWD_SJ; j++) {
-				const float o = (dkp_b + (int64_t)(s0 + j) * HW)[col];  // first tile: not written yet, not used
+				const float o = buf_load(rp, col_bytes, (unsigned)j * row_bytes);  // first tile: not written yet, not used
 				dk_old[j] = u > 0 ? o : 0.0f;
 			}
 		} else if (GROUPED && u > 0) {
@@ -590,11 +624,14 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			for (int j = 0; j < BWD_SJ; j++) dk_old[j] = (dkp_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
 		}
 		{
-			// all dA values of this step for the lane's head, read D float4 ahead of their use
+			// All dA values of this step for the lane's head, each float4 read D blocks ahead of its use, one read
+			// between two blocks of math.  Every instruction of a wave takes an issue slot, an s_waitcnt too: the
+			// branch-free form waits once per BL blocks instead of once per block (LDS reads return in order, so
+			// blocks bi..bi+BL-1 are there once no more than the D-BL+1 reads issued after them are outstanding).
 			const float4* gp0 = reinterpret_cast<const float4*>(gl + hl * TTP);
-			constexpr int NI4 = TT / 4, NBLK = BWD_SJ * NI4, D = FAST ? 2 : 1;
+			constexpr int NI4 = TT / 4, NBLK = BWD_SJ * NI4, BL = FAST ? BWD_LDS_BATCH : 1, D = 2 * BL - 1, RING = D + 1;
 			auto g_at = [&](int bi) { return gp0[((bi / NI4) * HB * TTP) / 4 + bi % NI4]; };
-			float4 g_ring[D + 1];
+			float4 g_ring[RING];
 #pragma unroll
 			for (int d = 0; d < D; d++) g_ring[d] = g_at(d);
 			// RANK: the tile values for the sums are read here and added up after the first src row's math,
@@ -609,19 +646,25 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 #pragma unroll
 				for (int m = 0; m < NM; m++) {
 					cs_v[m] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-					if (cs_row < BWD_SJ * HB && cs_sub + 16 * m < TT / 4) cs_v[m] = rp[cs_sub + 16 * m];
+					// FAST (64-token tiles, 64*HB threads): every group of sixteen lanes has a row, every lane a float4
+					if (FAST || (cs_row < BWD_SJ * HB && cs_sub + 16 * m < TT / 4)) cs_v[m] = rp[cs_sub + 16 * m];
 				}
 #pragma unroll
 				for (int n = 0; n < NR; n++) {
 #pragma unroll
-					for (int jj = 0; jj < BWD_SJ; jj++) rs_v[n][jj] = rs_lds[n] >= 0 ? gl[jj * HB * TTP + rs_lds[n]] : 0.0f;
+					for (int jj = 0; jj < BWD_SJ; jj++) rs_v[n][jj] = (FAST || rs_lds[n] >= 0) ? gl[jj * HB * TTP + rs_lds[n]] : 0.0f;
 				}
 			}
 #pragma unroll
 			for (int bi = 0; bi < NBLK; bi++) {
 				{
 					const int j = bi / NI4, i4 = bi % NI4;
-					if (bi + D < NBLK) g_ring[(bi + D) % (D + 1)] = g_at(bi + D);
+					if (bi + D < NBLK) g_ring[(bi + D) % RING] = g_at(bi + D);
+					if (BL > 1 && bi > 0 && bi % BL == 0) {
+						// s_waitcnt immediate: vmcnt and expcnt at their maxima, lgkmcnt in bits 11:8
+						if (bi + BL < NBLK) __builtin_amdgcn_s_waitcnt(0xC07F | ((D - BL + 1) << 8));
+						else __builtin_amdgcn_s_waitcnt(0xC07F);
+					}
 					__builtin_amdgcn_sched_barrier(0);
 					if (RANK && j == 1 && i4 == 0) {
 						// keep the loaded values opaque up to here, or the adds (and the wait for the loads)
@@ -639,17 +682,26 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 						for (int m = 0; m < NM; m++) a += (cs_v[m].x + cs_v[m].y) + (cs_v[m].z + cs_v[m].w);
 						a = row16_sum_to_last(a);
 						const int jj = cs_row / HB, s = s0 + jj;
-						if (cs_sub == 15 && cs_row < BWD_SJ * HB && (FAST || s < Tn)) csp_b[(int64_t)s * H + (cs_row - jj * HB)] = a;
+						if (cs_sub == 15 && (FAST || (cs_row < BWD_SJ * HB && s < Tn))) csp_b[(int64_t)s * H + (cs_row - jj * HB)] = a;
 #pragma unroll
 						for (int n = 0; n < NR; n++) rs_acc[n] += (rs_v[n][0] + rs_v[n][1]) + (rs_v[n][2] + rs_v[n][3]);
 						__builtin_amdgcn_sched_barrier(0);
 					}
-					if (RANK) pair_step4_rank(&qc[i4 * 4], kc[j], g_ring[bi % (D + 1)], &dqa[i4 * 4], dka[j]);
-					else pair_step4(&qc[i4 * 4], kc[j], g_ring[bi % (D + 1)], &dqa[i4 * 4], dka[j]);
+					if (RANK) pair_step4_rank(&qc[i4 * 4], kc[j], g_ring[bi % RING], &dqa[i4 * 4], dka[j]);
+					else pair_step4(&qc[i4 * 4], kc[j], g_ring[bi % RING], &dqa[i4 * 4], dka[j]);
 				}
 			}
 		}
 		settle();
+		if (FAST) {
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) {
+				const float v = RANK ? dka[j] : dka[j] * scale;
+				buf_store(GROUPED ? dk_old[j] + v : v, rp, col_bytes, (unsigned)j * row_bytes);
+			}
+			dkp_cur += (int64_t)BWD_SJ * HW;
+			continue;
+		}
 		// unconditional in the lane dimension: a store guarded by a per-lane predicate would let the
 		// compiler sink the dk chain into the guarded block and split the four-instruction groups
 #pragma unroll
@@ -918,7 +970,9 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.lds_bytes = (size_t)BWD_SJ * hb_max * (p.tt_rows + 4) * sizeof(float);
 	p.per = (int)l1_cdiv((int64_t)BWD_SJ * p.tt_rows * hb_max, p.threads);
 	if (p.lds_bytes > 64 * 1024 || p.per > 16 || (p.wide && p.per > 8)) { p.fast = false; return p; }
+	// (the branch-free form addresses a step's dA rows with 32-bit byte offsets from the step's first row)
 	p.branch_free = p.wide && p.tt_rows == 64 && T % 64 == 0 && T % BWD_SJ == 0 && HW % p.threads == 0 &&
+	                (BWD_SJ * T + 128) * H < ((int64_t)1 << 29) &&
 	                p.threads % W == 0 && (int64_t)BWD_SJ * 64 * (p.threads / W) == (int64_t)4 * p.threads;
 	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_groups * T * HW * sizeof(float) : 0;
 	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
