@@ -291,6 +291,33 @@ def test_dense_headline_size_properties():
     assert float((sq + sk).abs().max()) <= 1e-4 * float(sq.abs().max())
 
 
+def test_dense_more_than_2_31_logits():
+    """B=10 at the headline T, H, W: A and dA have 2.7e9 elements (10 GiB each), past 32-bit element and byte
+    offsets (the reference's PackedTensorAccessor32 cannot index them).  The batches are independent, so the
+    last batch must equal what a one-batch call gives: the forward bit for bit (every logit is one sum over
+    w), the backward to the gradient tolerance (a one-batch launch tiles differently)."""
+    print("case dense beyond 2^31 elements", flush=True)
+    B, T, H, W = 10, 4096, 16, 64
+    g = torch.Generator(device="cuda").manual_seed(31)
+    q = torch.randn(B, T, H, W, generator=g, device="cuda")
+    k = torch.randn(B, T, H, W, generator=g, device="cuda")
+    import _l1attn_hip as drv
+    a = drv.dense_forward(q, k)[0]
+    assert a.numel() > 2 ** 31
+    a1 = drv.dense_forward(q[B - 1:].contiguous(), k[B - 1:].contiguous())[0]
+    assert torch.equal(a[B - 1:], a1)
+    a0 = drv.dense_forward(q[:1].contiguous(), k[:1].contiguous())[0]
+    assert torch.equal(a[:1], a0)
+    del a0, a1
+    # use the logits as the upstream gradient: no second 10 GiB random tensor needed
+    dq, dk = drv.dense_backward(a, q, k)
+    dq1, dk1 = drv.dense_backward(a[B - 1:].contiguous(), q[B - 1:].contiguous(), k[B - 1:].contiguous())
+    assert cf.rel_err(dq[B - 1:].cpu(), dq1.cpu().double()) <= BWD_TOL
+    assert cf.rel_err(dk[B - 1:].cpu(), dk1.cpu().double()) <= BWD_TOL
+    sq, sk = dq.double().sum(1), dk.double().sum(1)
+    assert float((sq + sk).abs().max()) <= 1e-4 * float(sq.abs().max())
+
+
 @pytest.mark.parametrize("W", [16, 32, 33, 64, 65, 96, 97, 128])
 def test_dense_benchmark_grid_widths(W):
     """The widths of the reference's own timing sweep (benchmark.py:58-60), at two of its sequence lengths."""
