@@ -947,19 +947,21 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.tt_rows = p.wide ? 88 : 32;
 	p.group = 1;
 	if (p.wide) {
-		// One workgroup per CU at a time.  Pick the tile height and the tiles per workgroup that waste the
-		// least of the last round of workgroups; every partial array costs a write in the main kernel and
-		// a read in the reduction (0.04 tile rows per array, batch and column chunk, measured).
+		// Eight waves per CU at a time: one workgroup of 512 threads, two of 256.  Pick the tile height and the
+		// tiles per workgroup that waste the least of the last round of workgroups; every partial array costs
+		// a write in the main kernel and a read in the reduction (0.04 tile rows per array, batch and column
+		// chunk, measured).
 		double best = 1e30;
 		const int tr_max = p.rank ? 80 : 88;  // the rank variant keeps a few more values in registers
+		const int64_t slots = (int64_t)N_CU * (512 / p.threads);
 		for (int tr = 64; tr <= tr_max; tr += 8) {
 			for (int g = 1; g <= 8; g *= 2) {
 				const int64_t ngr = l1_cdiv(l1_cdiv(T, tr), g);
 				const int64_t wgs = B * p.n_cc * ngr;
 				// tiles are grouped only in the 64-token instantiations (registers), see launch_bwd_fast()
 				const int64_t per_tr = l1_cdiv((int64_t)BWD_SJ * tr * hb_exact, p.threads);
-				if (g > 1 && (wgs < N_CU || tr != 64 || per_tr > (p.rank ? 4 : 8))) continue;
-				const double cost = (double)l1_cdiv(wgs, N_CU) * g * (tr + 1.0) + 0.04 * (double)(B * p.n_cc * ngr);
+				if (g > 1 && (wgs < slots || tr != 64 || per_tr > (p.rank ? 4 : 8))) continue;
+				const double cost = (double)l1_cdiv(wgs, slots) * g * (tr + 1.0) + 0.04 * (double)(B * p.n_cc * ngr);
 				if (cost < best) { best = cost; p.tt_rows = tr; p.group = g; }
 			}
 		}
