@@ -365,6 +365,11 @@ __device__ __forceinline__ void buf_store(float v, buf_t r, unsigned lane_bytes,
 {
 	__builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, (int)lane_bytes, (int)uniform_bytes, 0);
 }
+// fp32 add in the L2, nothing returned
+__device__ __forceinline__ void buf_add(float v, buf_t r, unsigned lane_bytes, unsigned uniform_bytes)
+{
+	__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, r, (int)lane_bytes, (int)uniform_bytes, 0);
+}
 
 // Sum over each aligned group of 16 lanes (a DPP row); the total lands in the group's last lane.
 // Lanes shifted in from outside the row read as zero.
@@ -614,11 +619,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		for (int j = 0; j < BWD_SJ; j++) dk_old[j] = 0.0f;
 		const buf_t rp = make_buf(dkp_cur);
 		if (GROUPED && FAST) {
-#pragma unroll
-			for (int j = 0; j < BWD_SJ; j++) {
-				const float o = buf_load(rp, col_bytes, (unsigned)j * row_bytes);  // first tile: not written yet, not used
-				dk_old[j] = u > 0 ? o : 0.0f;
-			}
+			// nothing to load: the later tiles add to the stored rows in the L2 (below)
 		} else if (GROUPED && u > 0) {
 #pragma unroll
 			for (int j = 0; j < BWD_SJ; j++) dk_old[j] = (dkp_b + (int64_t)min(s0 + j, Tn - 1) * HW)[col];
@@ -694,10 +695,14 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		}
 		settle();
 		if (FAST) {
+			// GROUPED: the first tile stores, the others add in the L2: same lane, same address, tile order, so
+			// the sums are the same bits as a load, add and store would give, without the load and its wait
+			if (!GROUPED || u == 0) {
 #pragma unroll
-			for (int j = 0; j < BWD_SJ; j++) {
-				const float v = RANK ? dka[j] : dka[j] * scale;
-				buf_store(GROUPED ? dk_old[j] + v : v, rp, col_bytes, (unsigned)j * row_bytes);
+				for (int j = 0; j < BWD_SJ; j++) buf_store(RANK ? dka[j] : dka[j] * scale, rp, col_bytes, (unsigned)j * row_bytes);
+			} else {
+#pragma unroll
+				for (int j = 0; j < BWD_SJ; j++) buf_add(RANK ? dka[j] : dka[j] * scale, rp, col_bytes, (unsigned)j * row_bytes);
 			}
 			dkp_cur += (int64_t)BWD_SJ * HW;
 			continue;
