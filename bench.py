@@ -29,6 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per dense-backward launch (B=8,T=4096,H=16,W=64) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/dense_B8_T4096_H16_W64_pmc_*.txt), scaled by what three 1 GiB device copies read on the same
 # counters (profiles/copy_1GiB_pmc_*.txt: FETCH_SIZE 0.5 per KiB -> x2.0, WRITE_SIZE 1.0 per KiB -> x1.0).
+# (Counters collected before the later tiles' partial rows became L2 adds: the 6 GiB of them that the
+# workgroups read back are now read by the L2 instead; the total is unchanged to first order.)
 # KiB per kernel, fetch / write: column ranks 149986 / 262144, main kernel 10683411 / 8652097,
 # column-sum reduce 65547 / 2048, dk reduce 1050658 / 131072.
 DENSE_BWD_TRAFFIC_BYTES = ((149986 + 10683411 + 65547 + 1050658) * 2 + 262144 + 8652097 + 2048 + 131072) * 1024
