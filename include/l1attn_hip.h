@@ -72,8 +72,11 @@ int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn,
  * dk[b,s,h,w] = -sum_t scale*sign(q[b,t,h,w]-k[b,s,h,w]) * d_attn[b,s,t,h],   sign(0) = 0.
  * Replaces l1attn_cuda_drv.backward(d_attn,q,k) -> [dq,dk]  (cuda/l1attn_cuda_drv.cpp:67-104,
  * kernels cuda/l1attn_cuda_kernel.cu:206-455; CPU twin cpp/l1attn_drv.cpp:57-98).
- * d_attn is read in its native [B,S,T,H] layout.  Deterministic: no atomics; dk is summed
- * from per-dst-tile partials held in `workspace` (device memory, 256-byte aligned, at least
+ * d_attn is read in its native [B,S,T,H] layout.  Deterministic, unlike the reference's float
+ * atomics (cuda/l1attn_cuda_kernel.cu:439, :453): dk is summed in a fixed order from partial rows,
+ * each address of which is written by one lane only (where a workgroup adds several dst tiles into
+ * one partial, the additions are done by the L2 in that lane's program order).  The partials are
+ * held in `workspace` (device memory, 256-byte aligned, at least
  * l1attn_dense_bwd_workspace_bytes() for full speed; any multiple of one batch's share works,
  * the batches are then processed in several launches).  The f64 entry needs no workspace.
  * f32 fast path: sign() is taken from (q-k)*2^64, exact for |q|,|k| < 2^63 and differences
@@ -84,6 +87,20 @@ int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn,
  * sums (about 1e-6 of the largest gradient) instead of an exact zero.
  */
 size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W);
+/*
+ * No counterpart in the reference: reports how l1attn_dense_bwd_f32 tiles a shape, for tests of the host
+ * logic and for tuning; computes nothing on the GPU.  info[0..15]:
+ *   0 tiled path (else the generic kernels)   1 wide tiles (64..88 dst tokens, <= 512 threads)
+ *   2 column ranks                            3 branch-free step loop
+ *   4 threads per workgroup                   5 column chunks (workgroups across H*W)
+ *   6 dst tiles                               7 dst tokens per tile
+ *   8 staged d_attn values per thread, step   9 dst tiles per workgroup
+ *  10 workgroups along T (= partial arrays)  11 LDS bytes per workgroup
+ *  12 workspace bytes per batch              13 batches per launch with the full workspace
+ *  14, 15 reserved (0)
+ * Returns 0, or a negative argument error.
+ */
+int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64_t* info);
 int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk,
                          int64_t B, int64_t T, int64_t H, int64_t W,
                          void* workspace, size_t workspace_bytes, void* stream);

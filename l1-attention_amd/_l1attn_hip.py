@@ -44,6 +44,8 @@ def lib():
         L.l1attn_dense_fwd_ws_f32.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]
         L.l1attn_dense_bwd_workspace_bytes.restype = _c_sz
         L.l1attn_dense_bwd_workspace_bytes.argtypes = [_c_i64] * 4
+        L.l1attn_dense_bwd_plan_info.restype = ctypes.c_int
+        L.l1attn_dense_bwd_plan_info.argtypes = [_c_i64] * 4 + [_c_p]
         for sfx in ("f32", "f64"):
             f = getattr(L, "l1attn_dense_fwd_" + sfx)
             f.restype = ctypes.c_int

@@ -1116,6 +1116,22 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 	return p.per_batch_bytes * (size_t)nb;
 }
 
+int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64_t* info)
+{
+	if (!info || !shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	for (int i = 0; i < 16; i++) info[i] = 0;
+	if (B * T * H * W == 0) return L1ATTN_OK;
+	const BwdPlan p = bwd_plan(B, T, H, W);
+	info[0] = p.fast;
+	if (!p.fast) return L1ATTN_OK;
+	info[1] = p.wide; info[2] = p.rank; info[3] = p.branch_free;
+	info[4] = p.threads; info[5] = p.n_cc; info[6] = p.n_tt; info[7] = p.tt_rows;
+	info[8] = p.per; info[9] = p.group; info[10] = p.n_groups; info[11] = (int64_t)p.lds_bytes;
+	info[12] = (int64_t)p.per_batch_bytes;
+	info[13] = p.per_batch_bytes ? std::min<int64_t>(B, l1_cdiv(1024, (int64_t)p.n_groups * p.n_cc)) : B;
+	return L1ATTN_OK;
+}
+
 int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
                          int64_t T, int64_t H, int64_t W, void* workspace, size_t workspace_bytes, void* stream)
 {

@@ -72,6 +72,78 @@ def test_host_side_argument_logic(lib):
     assert lib.l1attn_expand_coo(None, 64, 2, 5, None, mx, None, 0, None) == -1    # null list
 
 
+def _plan(lib, B, T, H, W):
+    lib.l1attn_dense_bwd_plan_info.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_void_p]
+    a = (ctypes.c_int64 * 16)()
+    assert lib.l1attn_dense_bwd_plan_info(B, T, H, W, a) == 0
+    keys = ("tiled", "wide", "rank", "branch_free", "threads", "n_cc", "n_tt", "tt_rows", "per", "group", "n_groups",
+            "lds_bytes", "per_batch_bytes", "batches_per_launch")
+    return dict(zip(keys, list(a)))
+
+
+def test_dense_backward_plan_of_the_baseline_configurations(lib):
+    """How the three dense configurations of BASELINE.json are tiled (host logic only, no GPU)."""
+    c1 = _plan(lib, 2, 64, 4, 32)
+    assert c1["tiled"] and not c1["wide"] and not c1["rank"] and (c1["tt_rows"], c1["n_tt"], c1["threads"]) == (32, 2, 128)
+    c2 = _plan(lib, 16, 1024, 8, 64)
+    assert c2["wide"] and not c2["rank"] and c2["branch_free"]            # T < 2048: sign from the scaled difference
+    assert (c2["threads"], c2["n_cc"], c2["tt_rows"], c2["n_tt"], c2["group"]) == (512, 1, 64, 16, 1)  # 256 workgroups
+    c3 = _plan(lib, 8, 4096, 16, 64)
+    assert c3["wide"] and c3["rank"] and c3["branch_free"]
+    assert (c3["threads"], c3["n_cc"], c3["tt_rows"], c3["n_tt"], c3["group"], c3["n_groups"]) == (512, 2, 64, 64, 4, 16)
+    assert c3["batches_per_launch"] == 8 and c3["per"] == 4 and c3["lds_bytes"] == 4 * 8 * 68 * 4
+    # untiled shapes and empty problems
+    assert not _plan(lib, 2, 3, 16, 7)["tiled"]
+    assert _plan(lib, 0, 64, 4, 32) == {k: 0 for k in c1}
+    a = (ctypes.c_int64 * 16)()
+    assert lib.l1attn_dense_bwd_plan_info(1, -4, 2, 8, a) == -1 and lib.l1attn_dense_bwd_plan_info(1, 4, 2, 8, None) == -1
+
+
+def test_dense_backward_plan_invariants_over_a_shape_grid(lib):
+    """Every plan the host logic can produce on a grid of shapes must cover the problem exactly once and
+    respect what the kernels assume (threads, LDS, staged values, tile grouping, workspace size)."""
+    lib.l1attn_dense_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.l1attn_dense_bwd_workspace_bytes.argtypes = [ctypes.c_int64] * 4
+    cdiv = lambda a, b: -(-a // b)
+    seen = set()
+    for B in (1, 2, 3, 8, 16, 33):
+        for T in (16, 17, 64, 100, 512, 1000, 1024, 1536, 2048, 2100, 3000, 4096, 8192, 8200):
+            for H in (1, 2, 3, 4, 8, 12, 16, 32):
+                for W in (7, 16, 32, 33, 64, 96, 128):
+                    p = _plan(lib, B, T, H, W)
+                    HW = H * W
+                    if not p["tiled"]:
+                        assert T < 16 or HW < 32 or lib.l1attn_dense_bwd_workspace_bytes(B, T, H, W) == 0
+                        continue
+                    seen.add((p["wide"], p["rank"], p["branch_free"], p["group"] > 1))
+                    th = p["threads"]
+                    assert th % 64 == 0 and 64 <= th <= (512 if p["wide"] else 1024)
+                    assert (p["n_cc"] - 1) * th < HW <= p["n_cc"] * th
+                    assert p["n_tt"] == cdiv(T, p["tt_rows"]) and p["n_groups"] == cdiv(p["n_tt"], p["group"])
+                    assert p["tt_rows"] in ((64, 72, 80, 88) if p["wide"] else (32,))
+                    assert 0 < p["lds_bytes"] <= 64 * 1024 and 1 <= p["per"] <= (8 if p["wide"] else 16)
+                    heads = max(min(HW, (c + 1) * th) // W - (c * th) // W + (1 if min(HW, (c + 1) * th) % W else 0)
+                                for c in range(p["n_cc"]))
+                    assert p["per"] * th >= 4 * p["tt_rows"] * heads          # every staged value has a thread
+                    assert p["lds_bytes"] == 4 * heads * (p["tt_rows"] + 4) * 4
+                    if p["rank"]:
+                        assert p["wide"] and 2048 <= T <= 8192 and p["tt_rows"] <= 80 and 4 * heads * 16 <= th
+                    if p["group"] > 1:
+                        assert p["wide"] and p["tt_rows"] == 64 and p["per"] <= (4 if p["rank"] else 8)
+                        assert B * p["n_cc"] * p["n_groups"] >= 256 * (512 // th)
+                    if p["branch_free"]:
+                        assert p["wide"] and p["tt_rows"] == 64 and T % 64 == 0 and HW % th == 0 and W == 64 and p["per"] == 4
+                    partial = p["n_groups"] * T * HW * 4 if p["n_tt"] > 1 else 0
+                    ranks = (2 * T * HW + (p["n_tt"] + 1) * T * H) * 4 if p["rank"] else 0
+                    assert p["per_batch_bytes"] == partial + ranks
+                    nb = min(B, cdiv(1024, p["n_groups"] * p["n_cc"])) if p["per_batch_bytes"] else B
+                    assert p["batches_per_launch"] == nb
+                    assert lib.l1attn_dense_bwd_workspace_bytes(B, T, H, W) == p["per_batch_bytes"] * nb
+    # the grid reaches every family of instantiations: narrow, wide, ranks, branch-free, grouped
+    assert (0, 0, 0, False) in seen and (1, 0, 0, False) in seen and (1, 1, 0, False) in seen
+    assert (1, 1, 1, True) in seen and (1, 0, 1, True) in seen and (1, 1, 0, True) in seen
+
+
 def test_operator_modules_fail_loudly_without_library(monkeypatch):
     """No CPU or eager fallback: with the library missing the binding raises at first use."""
     import sys
