@@ -144,6 +144,20 @@ def test_dense_backward_plan_invariants_over_a_shape_grid(lib):
     assert (1, 1, 1, True) in seen and (1, 0, 1, True) in seen and (1, 1, 0, True) in seen
 
 
+def test_dense_forward_workspace_follows_the_width(lib):
+    """The forward needs scratch only for widths the tiled kernels cannot read directly: two zero-padded
+    copies [B,T,H,WP] with WP the next multiple of 16 (128 above 96); nothing for multiples of 16, for
+    widths above 128 or sequences below 32 tokens (generic kernels)."""
+    lib.l1attn_dense_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.l1attn_dense_fwd_workspace_bytes.argtypes = [ctypes.c_int64] * 4
+    B, T, H = 3, 100, 5
+    for W, WP in [(16, 0), (32, 0), (64, 0), (96, 0), (128, 0), (1, 16), (7, 16), (17, 32), (33, 48), (65, 80), (81, 96),
+                  (95, 96), (97, 128), (112, 0), (113, 128), (127, 128), (129, 0), (200, 0)]:
+        assert lib.l1attn_dense_fwd_workspace_bytes(B, T, H, W) == 2 * B * T * H * WP * 4, W
+    assert lib.l1attn_dense_fwd_workspace_bytes(B, 31, H, 33) == 0
+    assert lib.l1attn_dense_fwd_workspace_bytes(0, T, H, 33) == 0 and lib.l1attn_dense_fwd_workspace_bytes(B, T, H, -1) == 0
+
+
 def test_operator_modules_fail_loudly_without_library(monkeypatch):
     """No CPU or eager fallback: with the library missing the binding raises at first use."""
     import sys
