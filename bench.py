@@ -251,8 +251,9 @@ def main():
                          "kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the hot path does not communicate; "
-              "see DESIGN.md for how it would shard); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (the hot path does not communicate: batches and "
+              "heads are independent, so more GPUs would each take a share of them); run with --gpus 1",
+              file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():
