@@ -76,6 +76,59 @@ def check_scalar_prefetch(asm_text, kernel_substr="dense_fwd_f32_pipe"):
     return n_loads
 
 
+def kernel_resources(asm):
+    """Registers, scratch and LDS of every kernel in a device ISA listing, from its code-object metadata:
+    {mangled name: {"vgpr", "sgpr", "scratch_bytes", "lds_bytes", "vgpr_spills", "sgpr_spills"}}."""
+    fields = {".vgpr_count": "vgpr", ".sgpr_count": "sgpr", ".private_segment_fixed_size": "scratch_bytes",
+              ".group_segment_fixed_size": "lds_bytes", ".vgpr_spill_count": "vgpr_spills",
+              ".sgpr_spill_count": "sgpr_spills"}
+    out, cur = {}, {}
+    in_meta = False
+    for raw in asm.splitlines():
+        l = raw.strip()
+        if l.startswith("amdhsa.kernels:"):
+            in_meta = True
+            continue
+        if not in_meta:
+            continue
+        if l.startswith("- .") or l.startswith("amdhsa."):  # next kernel record, or the end of the list
+            if "name" in cur:
+                out[cur.pop("name")] = cur
+            cur = {}
+            l = l[2:] if l.startswith("- ") else l
+        key, _, val = l.partition(":")
+        key, val = key.strip(), val.strip()
+        if key == ".name":
+            cur["name"] = val
+        elif key in fields:
+            cur[fields[key]] = int(val)
+    if "name" in cur:
+        out[cur.pop("name")] = cur
+    return out
+
+
+def check_hot_kernels(res):
+    """The kernels of the headline path must run from registers: no scratch memory, no spilled VGPRs, and
+    a register count that leaves the waves per SIMD their launch geometry assumes."""
+    want = {  # substring of the mangled name -> most VGPRs per lane
+        "dense_fwd_f32_pipeILi64E": 128,                              # 1024 threads: four waves per SIMD
+        "dense_fwd_f32_pipeILi32E": 128,
+        "dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E": 256,        # 512 threads: two waves per SIMD
+        "dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1E": 256,
+        "dense_bwd_reduce_dkILb1ELb1E": 64,
+    }
+    problems = []
+    for sub, max_vgpr in want.items():
+        hits = [(n, r) for n, r in res.items() if sub in n]
+        if not hits:
+            problems.append("no kernel matches %s" % sub)
+        for n, r in hits:
+            if r.get("scratch_bytes", 0) or r.get("vgpr_spills", 0) or r.get("vgpr", 0) > max_vgpr:
+                problems.append("%s: %s" % (n, r))
+    if problems:
+        raise RuntimeError("hot-path kernels must not spill:\n" + "\n".join(problems))
+
+
 def build(verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = []
@@ -109,6 +162,11 @@ def build(verbose=False):
         raise RuntimeError("scalar-prefetch check found no pipelined forward kernel to verify")
     if verbose:
         print("scalar-prefetch check: %d loads verified" % n)
+    res = kernel_resources(asm)
+    check_hot_kernels(res)
+    with open(os.path.join(HERE, "build", "dense_kernel_resources.txt"), "w") as f:
+        for name in sorted(res):
+            f.write("%s %s\n" % (name, " ".join("%s=%d" % kv for kv in sorted(res[name].items()))))
     cmd = [hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd))

@@ -205,3 +205,55 @@ _ZN1_18dense_fwd_f32_pipeILi64EEEv: ; @k
         build.check_scalar_prefetch(good.replace("	s_waitcnt lgkmcnt(0)\n", ""))
     # kernels without the prefetch idiom are not inspected
     assert build.check_scalar_prefetch(good.replace("dense_fwd_f32_pipe", "other_kernel")) == 0
+
+
+def test_build_rejects_spills_in_the_hot_kernels():
+    """build.py reads registers and scratch of every dense kernel from the code-object metadata and fails
+    the build when a kernel of the headline path spills; the table of the last build is kept beside the
+    objects."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import build
+    meta = """
+amdhsa.kernels:
+  - .args:
+      - .offset: 0
+    .group_segment_fixed_size: 40960
+    .name:           _ZN1_18dense_fwd_f32_pipeILi64EEEv
+    .private_segment_fixed_size: 0
+    .sgpr_count:     100
+    .sgpr_spill_count: 1
+    .vgpr_count:     95
+    .vgpr_spill_count: 0
+  - .args:           []
+    .group_segment_fixed_size: 0
+    .name:           other_kernel
+    .private_segment_fixed_size: 344
+    .sgpr_count:     20
+    .vgpr_count:     128
+    .vgpr_spill_count: 12
+amdhsa.target:   amdgcn-amd-amdhsa--gfx950
+"""
+    res = build.kernel_resources(meta)
+    assert res["_ZN1_18dense_fwd_f32_pipeILi64EEEv"] == {"lds_bytes": 40960, "scratch_bytes": 0, "sgpr": 100,
+                                                         "sgpr_spills": 1, "vgpr": 95, "vgpr_spills": 0}
+    assert res["other_kernel"]["scratch_bytes"] == 344 and res["other_kernel"]["vgpr_spills"] == 12
+    full = {"k_dense_fwd_f32_pipeILi64E": dict(vgpr=95, scratch_bytes=0, vgpr_spills=0),
+            "k_dense_fwd_f32_pipeILi32E": dict(vgpr=70, scratch_bytes=0, vgpr_spills=0),
+            "k_dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E": dict(vgpr=218, scratch_bytes=0, vgpr_spills=0),
+            "k_dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1E": dict(vgpr=190, scratch_bytes=0, vgpr_spills=0),
+            "k_dense_bwd_reduce_dkILb1ELb1E": dict(vgpr=20, scratch_bytes=0, vgpr_spills=0)}
+    build.check_hot_kernels(full)
+    for name, change in [("k_dense_fwd_f32_pipeILi64E", dict(vgpr=130)),              # three waves per SIMD only
+                         ("k_dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E", dict(scratch_bytes=64)),
+                         ("k_dense_bwd_reduce_dkILb1ELb1E", dict(vgpr_spills=3))]:
+        bad = {k: dict(v) for k, v in full.items()}
+        bad[name].update(change)
+        with pytest.raises(RuntimeError, match="must not spill"):
+            build.check_hot_kernels(bad)
+    with pytest.raises(RuntimeError, match="no kernel matches"):
+        build.check_hot_kernels({k: v for k, v in full.items() if "reduce" not in k})
+    table = os.path.join(ROOT, "l1-attention_amd", "build", "dense_kernel_resources.txt")
+    if os.path.exists(table):  # written by the build that made the library under test
+        rows = open(table).read().splitlines()
+        assert any("dense_fwd_f32_pipeILi64E" in r and "scratch_bytes=0" in r for r in rows)
