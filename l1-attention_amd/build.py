@@ -130,6 +130,8 @@ def check_hot_kernels(res):
 
 
 def build(verbose=False):
+    sys.path.insert(0, HERE)
+    from isa_checks import check_forbidden  # a checker for the build machine only
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = []
     procs = []
@@ -143,6 +145,12 @@ def build(verbose=False):
             print(" ".join(cmd))
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
+    # device ISA listings of every source, for the checks below (in parallel with the compiles)
+    listings = []
+    for src in sources():
+        cmd = [hipcc, "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", "-I", os.path.join(HERE, "csrc"), "-S", "--cuda-device-only", src, "-o", "-"]
+        listings.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)))
     for src, p in procs:
         out, _ = p.communicate()
         # the host pass warns that it does not know the packed-fp32 feature; that is expected
@@ -151,12 +159,15 @@ def build(verbose=False):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if verbose and out.strip():
             print(out)
+    asm = None
+    for src, p in listings:
+        text, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError("hipcc -S failed on %s" % src)
+        check_forbidden(text, os.path.basename(src))  # isa_checks.py, imported below
+        if os.path.basename(src) == "dense.hip":
+            asm = text
     # ISA-level safety check of the kernels that prefetch through inline-asm scalar loads
-    dense = os.path.join(HERE, "csrc", "dense.hip")
-    asm = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-Xclang", "-target-feature",
-                          "-Xclang", "-packed-fp32-ops", "-I", os.path.join(HERE, "csrc"), "-S",
-                          "--cuda-device-only", dense, "-o", "-"],
-                         check=True, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True).stdout
     n = check_scalar_prefetch(asm)
     if n < 8:
         raise RuntimeError("scalar-prefetch check found no pipelined forward kernel to verify")
