@@ -138,9 +138,11 @@ def dense_backward(d_attn, q, k):
     check_input(d_attn, "d_attn")
     check_input(q, "q")
     check_input(k, "k")
+    if q.dim() != 4 or q.shape != k.shape or q.dtype != k.dtype or q.device != k.device:
+        raise RuntimeError("q and k must be [batch, n_ctx, n_heads, width] tensors of one shape, dtype and device")
     B, T, H, W = q.shape
-    if tuple(d_attn.shape) != (B, T, T, H) or d_attn.dtype != q.dtype:
-        raise RuntimeError("d_attn must be [batch, n_ctx, n_ctx, n_heads] with the dtype of q")
+    if tuple(d_attn.shape) != (B, T, T, H) or d_attn.dtype != q.dtype or d_attn.device != q.device:
+        raise RuntimeError("d_attn must be [batch, n_ctx, n_ctx, n_heads] with the dtype and device of q")
     sfx = sfx_of(q)
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
@@ -240,6 +242,19 @@ def _sparse_shapes(v, q, k):
     return B, T, H, W, v.shape[3]
 
 
+def _same_as(x, like, name, like_name):
+    if x.shape != like.shape or x.dtype != like.dtype or x.device != like.device:
+        raise RuntimeError("%s must have the shape, dtype and device of %s" % (name, like_name))
+
+
+def _edge_tensors(coo, P, q, E, B, H):
+    """coo (and the saved edge weights P, if given) must live on q's device; P is [batch, edges, heads]."""
+    if coo.device != q.device:
+        raise RuntimeError("coo must be on the device of q")
+    if P is not None and (tuple(P.shape) != (B, E, H) or P.dtype != q.dtype or P.device != q.device):
+        raise RuntimeError("attn must be the [batch, edges, heads] tensor the forward returned")
+
+
 def sparse_forward(v, q, k, coo, dst_mxlen, use_softmax, plan=None):
     """l1attn_sparse_cuda_drv.forward(v,q,k,coo,dst_mxlen,use_softmax) -> [vo, attn]
     (cuda/l1attn_sparse_cuda_drv.cpp:32-46).  The second tensor is the edge-weight tensor P [B,E,H]
@@ -248,6 +263,7 @@ def sparse_forward(v, q, k, coo, dst_mxlen, use_softmax, plan=None):
     for x, n in ((v, "v"), (q, "q"), (k, "k"), (coo, "coo")):
         check_input(x, n)
     B, T, H, W, Wv = _sparse_shapes(v, q, k)
+    _edge_tensors(coo, None, q, 0, B, H)
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
@@ -268,9 +284,11 @@ def sparse_backward(dvo, v, q, k, coo, P, dst_mxlen, use_softmax, plan=None):
     for x, n in ((dvo, "dvo"), (v, "v"), (q, "q"), (k, "k"), (coo, "coo"), (P, "attn")):
         check_input(x, n)
     B, T, H, W, Wv = _sparse_shapes(v, q, k)
+    _same_as(dvo, v, "dvo", "v")
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
+    _edge_tensors(coo, P, q, E, B, H)
     sfx = sfx_of(q)
     dv, dq, dk = torch.empty_like(v), torch.empty_like(q), torch.empty_like(k)
     DA = torch.empty_like(P)
@@ -287,8 +305,8 @@ def bidi_forward(vf, vb, q, k, coo, dst_mxlen, use_softmax, plan=None):
     for x, n in ((vf, "vf"), (vb, "vb"), (q, "q"), (k, "k"), (coo, "coo")):
         check_input(x, n)
     B, T, H, W, Wv = _sparse_shapes(vf, q, k)
-    if vb.shape != vf.shape or vb.dtype != vf.dtype:
-        raise RuntimeError("vf and vb must have one shape and dtype")
+    _same_as(vb, vf, "vb", "vf")
+    _edge_tensors(coo, None, q, 0, B, H)
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
@@ -308,9 +326,12 @@ def bidi_backward(dvo, vf, vb, q, k, coo, P, dst_mxlen, use_softmax, plan=None):
     for x, n in ((dvo, "dvo"), (vf, "vf"), (vb, "vb"), (q, "q"), (k, "k"), (coo, "coo"), (P, "attn")):
         check_input(x, n)
     B, T, H, W, Wv = _sparse_shapes(vf, q, k)
+    _same_as(vb, vf, "vb", "vf")
+    _same_as(dvo, vf, "dvo", "vf")
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
+    _edge_tensors(coo, P, q, E, B, H)
     sfx = sfx_of(q)
     dvf, dvb, dq, dk = torch.empty_like(vf), torch.empty_like(vb), torch.empty_like(q), torch.empty_like(k)
     DA = torch.empty_like(P)

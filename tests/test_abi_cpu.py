@@ -257,3 +257,99 @@ amdhsa.target:   amdgcn-amd-amdhsa--gfx950
     if os.path.exists(table):  # written by the build that made the library under test
         rows = open(table).read().splitlines()
         assert any("dense_fwd_f32_pipeILi64E" in r and "scratch_bytes=0" in r for r in rows)
+
+
+class _FakeLib(object):
+    """Stands in for the loaded library: every entry point accepts anything and reports success."""
+    def __getattr__(self, name):
+        if name.endswith("_bytes"):
+            return lambda *a: 256
+        if name == "l1attn_sparse_plan_check":
+            def chk(buf, E, T, hdr, st):
+                hdr[4], hdr[5] = 3, 2
+                return 0
+            return chk
+        return lambda *a: 0
+
+
+def test_driver_control_flow_without_a_gpu(monkeypatch):
+    """The Python drivers' argument checks, allocations and call sequences, walked on CPU tensors with the
+    library, the device checks and the stream lookup replaced by stand-ins (no kernel runs, no result is
+    looked at): a typing slip in a driver shows here and not only on the GPU box."""
+    import contextlib
+    import sys
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import _l1attn_hip as drv
+    monkeypatch.setattr(drv, "lib", lambda: _FakeLib())
+    monkeypatch.setattr(drv, "check_input", lambda x, name: None)
+    monkeypatch.setattr(drv, "stream_of", lambda x: None)
+    monkeypatch.setattr(torch.cuda, "device", lambda d: contextlib.nullcontext())
+    B, T, H, W, Wv, E = 2, 6, 3, 8, 4, 7
+    q, k = torch.zeros(B, T, H, W), torch.zeros(B, T, H, W)
+    v, vb = torch.zeros(B, T, H, Wv), torch.zeros(B, T, H, Wv)
+    coo = torch.zeros(E, 4, dtype=torch.int32)
+    a, = drv.dense_forward(q, k)
+    assert a.shape == (B, T, T, H)
+    dq, dk = drv.dense_backward(torch.zeros(B, T, T, H), q, k)
+    assert dq.shape == q.shape and dk.shape == k.shape
+    with pytest.raises(RuntimeError, match="d_attn must be"):
+        drv.dense_backward(torch.zeros(B, T, T, H + 1), q, k)
+    with pytest.raises(RuntimeError, match="one shape"):
+        drv.dense_backward(torch.zeros(B, T, T, H), q, torch.zeros(B, T, H, W + 1))
+    plan = drv.plan_for(coo, T)
+    assert (plan.E, plan.T, plan.max_dst_deg, plan.max_src_deg) == (E, T, 3, 2)
+    assert drv.plan_for(coo, T) is plan                      # cached on the tensor
+    coo[0, 0] = 1
+    assert drv.plan_for(coo, T) is not plan                  # in-place write invalidates
+    vo, P = drv.sparse_forward(v, q, k, coo, 3, True)
+    assert vo.shape == v.shape and P.shape == (B, E, H)
+    dv, dq, dk = drv.sparse_backward(torch.zeros_like(v), v, q, k, coo, P, 3, True)
+    assert dv.shape == v.shape and dq.shape == q.shape and dk.shape == k.shape
+    with pytest.raises(RuntimeError, match="dvo must have"):
+        drv.sparse_backward(torch.zeros(B, T, H, Wv + 1), v, q, k, coo, P, 3, True)
+    with pytest.raises(RuntimeError, match="attn must be"):
+        drv.sparse_backward(torch.zeros_like(v), v, q, k, coo, P[:, :-1], 3, True)
+    vo, P = drv.bidi_forward(v, vb, q, k, coo, 3, False)
+    assert vo.shape == v.shape and P.shape == (B, E, H)
+    grads = drv.bidi_backward(torch.zeros_like(v), v, vb, q, k, coo, P, 3, False)
+    assert [g.shape for g in grads] == [v.shape, vb.shape, q.shape, k.shape]
+    with pytest.raises(RuntimeError, match="vb must have"):
+        drv.bidi_forward(v, torch.zeros(B, T, H, Wv + 2), q, k, coo, 3, True)
+    with pytest.raises(RuntimeError, match="equal leading dims"):
+        drv.sparse_forward(torch.zeros(B, T + 1, H, Wv), q, k, coo, 3, True)
+    with pytest.raises(RuntimeError, match="only float32 and float64"):
+        drv.dense_forward(q.half(), k.half())
+
+
+def test_operator_modules_autograd_plumbing_without_a_gpu(monkeypatch):
+    """The three drop-in modules under autograd with the stand-in library: which tensors are saved, which
+    gradients come back (None for coo and the integers), five- and six-argument calls of the sparse module."""
+    import contextlib
+    import sys
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import _l1attn_hip as drv
+    import l1attn_cuda, l1attn_sparse_cuda, l1attn_sparse_bidi_cuda
+    monkeypatch.setattr(drv, "lib", lambda: _FakeLib())
+    monkeypatch.setattr(drv, "check_input", lambda x, name: None)
+    monkeypatch.setattr(drv, "stream_of", lambda x: None)
+    monkeypatch.setattr(torch.cuda, "device", lambda d: contextlib.nullcontext())
+    B, T, H, W, E = 2, 5, 3, 8, 6
+    mk = lambda *s: torch.zeros(*s, requires_grad=True)
+    q, k = mk(B, T, H, W), mk(B, T, H, W)
+    a = l1attn_cuda.L1Attn()(q, k)
+    assert a.shape == (B, T, T, H)
+    a.sum().backward()
+    assert q.grad.shape == q.shape and k.grad.shape == k.shape
+    coo = torch.zeros(E, 4, dtype=torch.int32)
+    v, q, k = mk(B, T, H, W), mk(B, T, H, W), mk(B, T, H, W)
+    m = l1attn_sparse_cuda.L1AttnSparse()
+    vo = m(v, q, k, coo, 2)                 # README form
+    vo2 = m(v, q, k, coo, 2, False)         # wrapper form
+    (vo.sum() + vo2.sum()).backward()
+    assert all(t.grad is not None and t.grad.shape == t.shape for t in (v, q, k))
+    vf, vb, q, k = mk(B, T, H, W), mk(B, T, H, W), mk(B, T, H, W), mk(B, T, H, W)
+    vo = l1attn_sparse_bidi_cuda.L1AttnSparseBidi()(vf, vb, q, k, coo, 2, True)
+    vo.sum().backward()
+    assert all(t.grad is not None and t.grad.shape == t.shape for t in (vf, vb, q, k))
