@@ -696,7 +696,8 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		settle();
 		if (FAST) {
 			// GROUPED: the first tile stores, the others add in the L2: same lane, same address, tile order, so
-			// the sums are the same bits as a load, add and store would give, without the load and its wait
+			// the sums are formed in the order a load, add and store would form them (and repeat bit for bit),
+			// without the load and its wait
 			if (!GROUPED || u == 0) {
 #pragma unroll
 				for (int j = 0; j < BWD_SJ; j++) buf_store(RANK ? dka[j] : dka[j] * scale, rp, col_bytes, (unsigned)j * row_bytes);
