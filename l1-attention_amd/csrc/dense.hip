@@ -960,13 +960,18 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 		double best = 1e30;
 		const int tr_max = p.rank ? 80 : 88;  // the rank variant keeps a few more values in registers
 		const int64_t slots = (int64_t)N_CU * (512 / p.threads);
+		// tiles are grouped only where the branch-free step loop runs (whole 64-token tiles, whole column
+		// chunks, heads of 64 columns): that is the form whose later tiles add to the partial in the L2
+		const bool can_group = T % 64 == 0 && T % BWD_SJ == 0 && HW % p.threads == 0 && p.threads % W == 0 &&
+		                       (int64_t)BWD_SJ * 64 * (p.threads / W) == (int64_t)4 * p.threads &&
+		                       (BWD_SJ * T + 128) * H < ((int64_t)1 << 29);
 		for (int tr = 64; tr <= tr_max; tr += 8) {
 			for (int g = 1; g <= 8; g *= 2) {
 				const int64_t ngr = l1_cdiv(l1_cdiv(T, tr), g);
 				const int64_t wgs = B * p.n_cc * ngr;
 				// tiles are grouped only in the 64-token instantiations (registers), see launch_bwd_fast()
 				const int64_t per_tr = l1_cdiv((int64_t)BWD_SJ * tr * hb_exact, p.threads);
-				if (g > 1 && (wgs < slots || tr != 64 || per_tr > (p.rank ? 4 : 8))) continue;
+				if (g > 1 && (!can_group || wgs < slots || tr != 64 || per_tr > (p.rank ? 4 : 8))) continue;
 				const double cost = (double)l1_cdiv(wgs, slots) * g * (tr + 1.0) + 0.04 * (double)(B * p.n_cc * ngr);
 				if (cost < best) { best = cost; p.tt_rows = tr; p.group = g; }
 			}
@@ -1002,11 +1007,6 @@ void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* d
 		else if (p.rank) L1_BWD_CASE6(64, 512, 4, true, false, true);
 		else if (p.group > 1) L1_BWD_CASE6(64, 512, 4, false, true, true);
 		else L1_BWD_CASE6(64, 512, 4, false, false, true);
-	} else if (p.wide && p.group > 1) {
-		// bwd_plan() groups tiles only for these instantiations
-		if (p.rank) L1_BWD_CASE(64, 512, 4, true, true);
-		else if (p.per <= 4) L1_BWD_CASE(64, 512, 4, false, true);
-		else L1_BWD_CASE(64, 512, 8, false, true);
 	} else if (p.wide && p.rank) {
 		switch (p.tt_rows) {
 		case 64:

@@ -130,6 +130,7 @@ def test_dense_backward_plan_invariants_over_a_shape_grid(lib):
                         assert p["wide"] and 2048 <= T <= 8192 and p["tt_rows"] <= 80 and 4 * heads * 16 <= th
                     if p["group"] > 1:
                         assert p["wide"] and p["tt_rows"] == 64 and p["per"] <= (4 if p["rank"] else 8)
+                        assert p["branch_free"]                               # grouped tiles only in the branch-free form
                         assert B * p["n_cc"] * p["n_groups"] >= 256 * (512 // th)
                     if p["branch_free"]:
                         assert p["wide"] and p["tt_rows"] == 64 and T % 64 == 0 and HW % th == 0 and W == 64 and p["per"] == 4
@@ -141,7 +142,8 @@ def test_dense_backward_plan_invariants_over_a_shape_grid(lib):
                     assert lib.l1attn_dense_bwd_workspace_bytes(B, T, H, W) == p["per_batch_bytes"] * nb
     # the grid reaches every family of instantiations: narrow, wide, ranks, branch-free, grouped
     assert (0, 0, 0, False) in seen and (1, 0, 0, False) in seen and (1, 1, 0, False) in seen
-    assert (1, 1, 1, True) in seen and (1, 0, 1, True) in seen and (1, 1, 0, True) in seen
+    assert (1, 1, 1, True) in seen and (1, 0, 1, True) in seen and (1, 1, 1, False) in seen and (1, 0, 1, False) in seen
+    assert not any(grouped and not bf for (_, _, bf, grouped) in seen)
 
 
 def test_dense_forward_workspace_follows_the_width(lib):

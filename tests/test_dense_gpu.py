@@ -182,7 +182,7 @@ def _with_ties(q, k, seed):
                                        ((8, 1024, 32, 64), "the same with two dst tiles per workgroup"),
                                        ((5, 1102, 32, 64), "wide tiles, ragged T (general step loop)"),
                                        ((3, 2048, 32, 64), "wide tiles, sign from column ranks"),
-                                       ((4, 2100, 32, 64), "ranks, two dst tiles per workgroup, ragged last group")])
+                                       ((4, 2100, 32, 64), "ranks, 72-token tiles, ragged T (general step loop)")])
 def test_dense_backward_long_sequences_vs_oracle(shape, tag):
     """The two backward paths for long sequences (dst tiles of 64..88 tokens; for T >= 2048 on column
     ranks), with planted ties, against the oracle."""
