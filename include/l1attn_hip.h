@@ -234,6 +234,35 @@ int l1attn_sparse_bidi_bwd_f64(const double* dvo, const double* vf, const double
                                int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
                                int use_softmax, void* stream);
 
+/*
+ * The two forwards with 16-bit rows: v/vf, vb, q, k and vo are IEEE binary16 (f16) or bfloat16
+ * (bf16) in memory, 2 bytes per element, in the layouts above.  Logits, softmax and value sums run
+ * in fp32; vo is rounded to nearest even once on store (bidi: once after the dst pass and once
+ * after the src pass adds its sum); P [B,E,H] is fp32.  Same limits and return codes as the f32
+ * entry points; 16-byte aligned pointers with W and Wv multiples of 4 take the vector path.
+ * Replaces the Half instantiation of the reference's forward launchers
+ * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, cuda/l1attn_sparse_cuda_kernel.cu:405-435 and :684-714),
+ * which computes every step in half precision.  There is no 16-bit backward, as in the reference:
+ * its backward launchers dispatch float and double only (:483-519, :765-803).  bfloat16 is an
+ * addition.
+ */
+int l1attn_sparse_fwd_f16(const void* v, const void* q, const void* k, const void* plan,
+                          void* vo, float* P,
+                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                          int use_softmax, void* stream);
+int l1attn_sparse_fwd_bf16(const void* v, const void* q, const void* k, const void* plan,
+                           void* vo, float* P,
+                           int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                           int use_softmax, void* stream);
+int l1attn_sparse_bidi_fwd_f16(const void* vf, const void* vb, const void* q, const void* k,
+                               const void* plan, void* vo, float* P,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                               int use_softmax, void* stream);
+int l1attn_sparse_bidi_fwd_bf16(const void* vf, const void* vb, const void* q, const void* k,
+                                const void* plan, void* vo, float* P,
+                                int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                                int use_softmax, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -74,6 +74,11 @@ def lib():
                 f = getattr(L, name + sfx)
                 f.restype = _c_i
                 f.argtypes = [_c_p] * nptr + dims
+        for sfx in ("f16", "bf16"):  # forward only, as in the reference
+            for name, nptr in (("l1attn_sparse_fwd_", 6), ("l1attn_sparse_bidi_fwd_", 7)):
+                f = getattr(L, name + sfx)
+                f.restype = _c_i
+                f.argtypes = [_c_p] * nptr + dims
         _lib = L
     return _lib
 
@@ -100,6 +105,26 @@ def sfx_of(x, name="q"):
     if x.dtype == torch.float64:
         return "f64"
     raise RuntimeError("%s: only float32 and float64 are implemented, got %s" % (name, x.dtype))
+
+
+def sfx_fwd_sparse(x, name="q"):
+    """Entry-point suffix and edge-weight dtype of the sparse forwards.  They also take 16-bit rows
+    (the reference dispatches Half there: cuda/l1attn_sparse_cuda_kernel.cu:405-435, :684-714);
+    the weights of a 16-bit forward are fp32."""
+    if x.dtype == torch.float16:
+        return "f16", torch.float32
+    if x.dtype == torch.bfloat16:
+        return "bf16", torch.float32
+    return sfx_of(x, name), x.dtype
+
+
+def sfx_bwd_sparse(x):
+    """The sparse backwards exist for float32 and float64 only, like the reference's
+    (AT_DISPATCH_FLOATING_TYPES, cuda/l1attn_sparse_cuda_kernel.cu:483-519, :765-803)."""
+    if x.dtype in (torch.float16, torch.bfloat16):
+        raise RuntimeError("the sparse backward is not implemented for %s (forward only, as in the reference)"
+                           % x.dtype)
+    return sfx_of(x)
 
 
 def stream_of(x):
@@ -267,9 +292,9 @@ def sparse_forward(v, q, k, coo, dst_mxlen, use_softmax, plan=None):
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
-    sfx = sfx_of(q)
+    sfx, p_dtype = sfx_fwd_sparse(q)
     vo = torch.empty_like(v)
-    P = torch.empty((B, E, H), dtype=q.dtype, device=q.device)
+    P = torch.empty((B, E, H), dtype=p_dtype, device=q.device)
     with torch.cuda.device(q.device):
         rc = getattr(lib(), "l1attn_sparse_fwd_" + sfx)(
             ptr(v), ptr(q), ptr(k), ptr(plan.buf), ptr(vo), ptr(P), B, T, H, W, Wv, E,
@@ -284,12 +309,12 @@ def sparse_backward(dvo, v, q, k, coo, P, dst_mxlen, use_softmax, plan=None):
     for x, n in ((dvo, "dvo"), (v, "v"), (q, "q"), (k, "k"), (coo, "coo"), (P, "attn")):
         check_input(x, n)
     B, T, H, W, Wv = _sparse_shapes(v, q, k)
+    sfx = sfx_bwd_sparse(q)
     _same_as(dvo, v, "dvo", "v")
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
     _edge_tensors(coo, P, q, E, B, H)
-    sfx = sfx_of(q)
     dv, dq, dk = torch.empty_like(v), torch.empty_like(q), torch.empty_like(k)
     DA = torch.empty_like(P)
     with torch.cuda.device(q.device):
@@ -310,9 +335,9 @@ def bidi_forward(vf, vb, q, k, coo, dst_mxlen, use_softmax, plan=None):
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
-    sfx = sfx_of(q)
+    sfx, p_dtype = sfx_fwd_sparse(q)
     vo = torch.empty_like(vf)
-    P = torch.empty((B, E, H), dtype=q.dtype, device=q.device)
+    P = torch.empty((B, E, H), dtype=p_dtype, device=q.device)
     with torch.cuda.device(q.device):
         rc = getattr(lib(), "l1attn_sparse_bidi_fwd_" + sfx)(
             ptr(vf), ptr(vb), ptr(q), ptr(k), ptr(plan.buf), ptr(vo), ptr(P), B, T, H, W, Wv, E,
@@ -326,13 +351,13 @@ def bidi_backward(dvo, vf, vb, q, k, coo, P, dst_mxlen, use_softmax, plan=None):
     for x, n in ((dvo, "dvo"), (vf, "vf"), (vb, "vb"), (q, "q"), (k, "k"), (coo, "coo"), (P, "attn")):
         check_input(x, n)
     B, T, H, W, Wv = _sparse_shapes(vf, q, k)
+    sfx = sfx_bwd_sparse(q)
     _same_as(vb, vf, "vb", "vf")
     _same_as(dvo, vf, "dvo", "vf")
     if plan is None:
         plan = plan_for(coo, T)
     E = plan.E
     _edge_tensors(coo, P, q, E, B, H)
-    sfx = sfx_of(q)
     dvf, dvb, dq, dk = torch.empty_like(vf), torch.empty_like(vb), torch.empty_like(q), torch.empty_like(k)
     DA = torch.empty_like(P)
     with torch.cuda.device(q.device):

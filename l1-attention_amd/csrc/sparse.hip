@@ -22,33 +22,54 @@
 
 namespace {
 
-template <typename T, int VEC>
-__device__ __forceinline__ void ldv(const T* __restrict__ p, T (&x)[VEC])
+// Storage types of the 16-bit forward entry points: IEEE half and bfloat16.  Rows are held in memory in
+// the storage type S and converted on load and on store; every sum runs in the compute type T (float).
+using f16_t = _Float16;
+using bf16_t = __bf16;
+
+// x[0..VEC) = the VEC consecutive elements at p, converted from S to T.  VEC == 4 takes one 16-byte
+// (float), two 16-byte (double) or one 8-byte (16-bit types) access; p is aligned to that by the host.
+template <typename T, int VEC, typename S>
+__device__ __forceinline__ void ldv(const S* __restrict__ p, T (&x)[VEC])
 {
-	if constexpr (VEC == 4 && sizeof(T) == 4) {
+	if constexpr (VEC == 4 && sizeof(S) == 4) {
 		const float4 t = *reinterpret_cast<const float4*>(p);
 		x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
-	} else if constexpr (VEC == 4 && sizeof(T) == 8) {
+	} else if constexpr (VEC == 4 && sizeof(S) == 8) {
 		const double2 a = *reinterpret_cast<const double2*>(p);
 		const double2 b = *reinterpret_cast<const double2*>(p + 2);
 		x[0] = a.x; x[1] = a.y; x[2] = b.x; x[3] = b.y;
+	} else if constexpr (VEC == 4 && sizeof(S) == 2) {
+		const uint2 raw = *reinterpret_cast<const uint2*>(p);
+		S h[4];
+		__builtin_memcpy(h, &raw, 8);
+#pragma unroll
+		for (int i = 0; i < 4; i++) x[i] = (T)h[i];
 	} else {
 #pragma unroll
-		for (int i = 0; i < VEC; i++) x[i] = p[i];
+		for (int i = 0; i < VEC; i++) x[i] = (T)p[i];
 	}
 }
 
-template <typename T, int VEC>
-__device__ __forceinline__ void stv(T* __restrict__ p, const T (&x)[VEC])
+// the VEC consecutive elements at p = x[0..VEC), rounded to S (round to nearest even for the 16-bit types)
+template <typename T, int VEC, typename S>
+__device__ __forceinline__ void stv(S* __restrict__ p, const T (&x)[VEC])
 {
-	if constexpr (VEC == 4 && sizeof(T) == 4) {
+	if constexpr (VEC == 4 && sizeof(S) == 4) {
 		*reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
-	} else if constexpr (VEC == 4 && sizeof(T) == 8) {
+	} else if constexpr (VEC == 4 && sizeof(S) == 8) {
 		*reinterpret_cast<double2*>(p) = make_double2(x[0], x[1]);
 		*reinterpret_cast<double2*>(p + 2) = make_double2(x[2], x[3]);
+	} else if constexpr (VEC == 4 && sizeof(S) == 2) {
+		S h[4];
+#pragma unroll
+		for (int i = 0; i < 4; i++) h[i] = (S)x[i];
+		uint2 raw;
+		__builtin_memcpy(&raw, h, 8);
+		*reinterpret_cast<uint2*>(p) = raw;
 	} else {
 #pragma unroll
-		for (int i = 0; i < VEC; i++) p[i] = x[i];
+		for (int i = 0; i < VEC; i++) p[i] = (S)x[i];
 	}
 }
 
@@ -155,11 +176,12 @@ template <int MC> struct Unroll { static constexpr int EU = MC == 1 ? 4 : 1; };
 // ---------------------------------------------------------------------------------- forward
 
 // dst pass: logits, softmax with the "+1" denominator, value sum.  Writes vo rows and P.
-template <typename T, int VEC, int MC, int NWV>
+// S: type of the rows in memory (v, q, k, vo); T: type of the sums and of the weights P.
+template <typename T, int VEC, int MC, int NWV, typename S>
 __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_dst(
-    const T* __restrict__ v, const T* __restrict__ q, const T* __restrict__ k, const int* __restrict__ dst_ptr,
+    const S* __restrict__ v, const S* __restrict__ q, const S* __restrict__ k, const int* __restrict__ dst_ptr,
     const int* __restrict__ csr_src, const int* __restrict__ long_list, const int* __restrict__ n_long,
-    T* __restrict__ vo, T* __restrict__ P, Geo g, int use_softmax, T scale)
+    S* __restrict__ vo, T* __restrict__ P, Geo g, int use_softmax, T scale)
 {
 	extern __shared__ unsigned char smem_raw[];
 	T* smem = reinterpret_cast<T*>(smem_raw);
@@ -168,9 +190,9 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_dst(
 	if (!wave_item<NWV>(g, dst_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowq = (int64_t)g.H * g.W, rowv = (int64_t)g.H * g.Wv;
-	const T* qb = q + (int64_t)b * g.Tn * rowq;
-	const T* kb = k + (int64_t)b * g.Tn * rowq;
-	const T* vb = v + (int64_t)b * g.Tn * rowv;
+	const S* qb = q + (int64_t)b * g.Tn * rowq;
+	const S* kb = k + (int64_t)b * g.Tn * rowq;
+	const S* vb = v + (int64_t)b * g.Tn * rowv;
 	T* Pb = P + (int64_t)b * g.E * g.H;
 
 	T qv[MC][VEC], acc[MC][VEC];
@@ -254,11 +276,11 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_dst(
 }
 
 // bidi src pass: vo[b,src] += sum over the src's edges of p * vb[b,dst]   (cpp/l1attn_sparse_bidi_drv.cpp:93-96)
-template <typename T, int VEC, int MC, int NWV>
+template <typename T, int VEC, int MC, int NWV, typename S>
 __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_src(
-    const T* __restrict__ vbk, const int* __restrict__ src_ptr, const int* __restrict__ csc_dst,
+    const S* __restrict__ vbk, const int* __restrict__ src_ptr, const int* __restrict__ csc_dst,
     const int* __restrict__ csc_slot, const int* __restrict__ long_list, const int* __restrict__ n_long,
-    const T* __restrict__ P, T* __restrict__ vo, Geo g)
+    const T* __restrict__ P, S* __restrict__ vo, Geo g)
 {
 	extern __shared__ unsigned char smem_raw[];
 	T* smem = reinterpret_cast<T*>(smem_raw);
@@ -267,7 +289,7 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_src(
 	if (!wave_item<NWV>(g, src_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowv = (int64_t)g.H * g.Wv;
-	const T* vb = vbk + (int64_t)b * g.Tn * rowv;
+	const S* vb = vbk + (int64_t)b * g.Tn * rowv;
 	const T* Pb = P + (int64_t)b * g.E * g.H;
 	T acc[MC][VEC];
 	bool okv[MC];
@@ -320,7 +342,7 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_src(
 #pragma unroll
 		for (int m = 0; m < MC; m++) {
 			if (okv[m]) {
-				T* o = vo + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m];
+				S* o = vo + ((int64_t)b * g.Tn + L.tok) * rowv + offv[m];
 				T y[VEC];
 				ldv<T, VEC>(o, y);
 #pragma unroll
@@ -614,8 +636,8 @@ int make_cfg(const Shape& s, const void* plan, const void* const* ptrs, int n_pt
 		}                                                                                  \
 	} while (0)
 
-template <typename T>
-int sparse_fwd_impl(const T* v, const T* vbk, const T* q, const T* k, const void* plan, T* vo, T* P, Shape s,
+template <typename T, typename S>
+int sparse_fwd_impl(const S* v, const S* vbk, const S* q, const S* k, const void* plan, S* vo, T* P, Shape s,
                     int use_softmax, bool bidi, hipStream_t st)
 {
 	if (s.B * s.T * s.H == 0) return L1ATTN_OK;
@@ -626,14 +648,14 @@ int sparse_fwd_impl(const T* v, const T* vbk, const T* q, const T* k, const void
 	if (rc) return rc;
 	const T scale = (T)(-1.0 / sqrt((double)s.W));
 #define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
-	hipLaunchKernelGGL((sparse_fwd_dst<T, V, M, N>), GRID, BLOCK, LDS, st, v, q, k, c.dst_ptr, c.csr_src,        \
+	hipLaunchKernelGGL((sparse_fwd_dst<T, V, M, N, S>), GRID, BLOCK, LDS, st, v, q, k, c.dst_ptr, c.csr_src,        \
 	                   c.long_dst, c.n_long_dst, vo, P, c.g, use_softmax, scale)
 	DISPATCH_VM(c, T, CALL);
 #undef CALL
 	L1_LAUNCH_CHECK();
 	if (bidi) {
 #define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
-	hipLaunchKernelGGL((sparse_fwd_src<T, V, M, N>), GRID, BLOCK, LDS, st, vbk, c.src_ptr, c.csc_dst,            \
+	hipLaunchKernelGGL((sparse_fwd_src<T, V, M, N, S>), GRID, BLOCK, LDS, st, vbk, c.src_ptr, c.csc_dst,            \
 	                   c.csc_slot, c.long_src, c.n_long_src, (const T*)P, vo, c.g)
 		DISPATCH_VM(c, T, CALL);
 #undef CALL
@@ -686,7 +708,7 @@ extern "C" {
 	                            int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E, int use_softmax, \
 	                            void* stream)                                                                       \
 	{                                                                                                               \
-		return sparse_fwd_impl<TYPE>(v, nullptr, q, k, plan, vo, P, Shape{B, T, H, W, Wv, E}, use_softmax, false,   \
+		return sparse_fwd_impl<TYPE, TYPE>(v, nullptr, q, k, plan, vo, P, Shape{B, T, H, W, Wv, E}, use_softmax, false,   \
 		                             (hipStream_t)stream);                                                          \
 	}                                                                                                               \
 	int l1attn_sparse_bwd_##SFX(const TYPE* dvo, const TYPE* v, const TYPE* q, const TYPE* k, const void* plan,     \
@@ -700,7 +722,7 @@ extern "C" {
 	                                 const void* plan, TYPE* vo, TYPE* P, int64_t B, int64_t T, int64_t H,          \
 	                                 int64_t W, int64_t Wv, int64_t E, int use_softmax, void* stream)               \
 	{                                                                                                               \
-		return sparse_fwd_impl<TYPE>(vf, vb, q, k, plan, vo, P, Shape{B, T, H, W, Wv, E}, use_softmax, true,        \
+		return sparse_fwd_impl<TYPE, TYPE>(vf, vb, q, k, plan, vo, P, Shape{B, T, H, W, Wv, E}, use_softmax, true,        \
 		                             (hipStream_t)stream);                                                          \
 	}                                                                                                               \
 	int l1attn_sparse_bidi_bwd_##SFX(const TYPE* dvo, const TYPE* vf, const TYPE* vb, const TYPE* q,                \
@@ -714,5 +736,30 @@ extern "C" {
 
 L1_SPARSE_ENTRY(f32, float)
 L1_SPARSE_ENTRY(f64, double)
+
+// Forward only with 16-bit rows (the reference dispatches its forward kernels for Half as well,
+// cuda/l1attn_sparse_cuda_kernel.cu:405-435 and :684-714, and its backward kernels for float and double
+// only, :483-519): v, q, k and vo are IEEE half (f16) or bfloat16 (bf16) in memory, the logits, the
+// softmax and the value sums run in fp32, the weights P are fp32.
+#define L1_SPARSE_FWD16_ENTRY(SFX, STYPE)                                                                           \
+	int l1attn_sparse_fwd_##SFX(const void* v, const void* q, const void* k, const void* plan, void* vo, float* P,   \
+	                            int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E, int use_softmax, \
+	                            void* stream)                                                                       \
+	{                                                                                                               \
+		return sparse_fwd_impl<float, STYPE>((const STYPE*)v, nullptr, (const STYPE*)q, (const STYPE*)k, plan,      \
+		                                     (STYPE*)vo, P, Shape{B, T, H, W, Wv, E}, use_softmax, false,           \
+		                                     (hipStream_t)stream);                                                  \
+	}                                                                                                               \
+	int l1attn_sparse_bidi_fwd_##SFX(const void* vf, const void* vb, const void* q, const void* k,                  \
+	                                 const void* plan, void* vo, float* P, int64_t B, int64_t T, int64_t H,         \
+	                                 int64_t W, int64_t Wv, int64_t E, int use_softmax, void* stream)               \
+	{                                                                                                               \
+		return sparse_fwd_impl<float, STYPE>((const STYPE*)vf, (const STYPE*)vb, (const STYPE*)q, (const STYPE*)k,  \
+		                                     plan, (STYPE*)vo, P, Shape{B, T, H, W, Wv, E}, use_softmax, true,      \
+		                                     (hipStream_t)stream);                                                  \
+	}
+
+L1_SPARSE_FWD16_ENTRY(f16, f16_t)
+L1_SPARSE_FWD16_ENTRY(bf16, bf16_t)
 
 }  // extern "C"

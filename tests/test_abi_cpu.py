@@ -262,8 +262,12 @@ amdhsa.target:   amdgcn-amd-amdhsa--gfx950
 
 
 class _FakeLib(object):
-    """Stands in for the loaded library: every entry point accepts anything and reports success."""
+    """Stands in for the loaded library: every entry point accepts anything and reports success.
+    `calls` lists the names looked up, in order."""
+    calls = []
+
     def __getattr__(self, name):
+        _FakeLib.calls.append(name)
         if name.endswith("_bytes"):
             return lambda *a: 256
         if name == "l1attn_sparse_plan_check":
@@ -322,6 +326,22 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
         drv.sparse_forward(torch.zeros(B, T + 1, H, Wv), q, k, coo, 3, True)
     with pytest.raises(RuntimeError, match="only float32 and float64"):
         drv.dense_forward(q.half(), k.half())
+    # 16-bit rows: forward only, fp32 edge weights, the entry point named after the storage type
+    for dt, sfx in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+        v16, vb16, q16, k16 = (x.to(dt) for x in (v, vb, q, k))
+        del _FakeLib.calls[:]
+        vo, P = drv.sparse_forward(v16, q16, k16, coo, 3, True)
+        assert _FakeLib.calls[-1] == "l1attn_sparse_fwd_" + sfx
+        assert vo.dtype == dt and vo.shape == v.shape and P.dtype == torch.float32 and P.shape == (B, E, H)
+        vo, P = drv.bidi_forward(v16, vb16, q16, k16, coo, 3, False)
+        assert _FakeLib.calls[-1] == "l1attn_sparse_bidi_fwd_" + sfx
+        assert vo.dtype == dt and P.dtype == torch.float32
+        with pytest.raises(RuntimeError, match="backward is not implemented"):
+            drv.sparse_backward(torch.zeros_like(v16), v16, q16, k16, coo, P, 3, True)
+        with pytest.raises(RuntimeError, match="backward is not implemented"):
+            drv.bidi_backward(torch.zeros_like(v16), v16, vb16, q16, k16, coo, P, 3, True)
+        with pytest.raises(RuntimeError, match="share dtype"):
+            drv.sparse_forward(v, q16, k16, coo, 3, True)
 
 
 def test_operator_modules_autograd_plumbing_without_a_gpu(monkeypatch):
