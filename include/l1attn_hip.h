@@ -120,6 +120,24 @@ int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k,
 int l1attn_dense_column_ranks_f32(const float* q, const float* k, float* rq, float* rk,
                                   int64_t B, int64_t T, int64_t H, int64_t W, void* stream);
 
+/*
+ * Fused forward: dense L1 logits, softmax over the src tokens with the no-op zero logit, value sum;
+ * the [B,S,T,H] logits are never written.
+ *   a[s]        = -1/sqrt(W) * sum_w |q[b,t,h,w] - k[b,s,h,w]|
+ *   vo[b,t,h,:] = sum_s exp(a[s]) * v[b,s,h,:] / (1 + sum_s exp(a[s]))
+ *   lse[b,t,h]  = log(1 + sum_s exp(a[s]))          (optional: lse may be NULL)
+ * The reference has no single function for this; it is the composition its model code builds from
+ * l1attn_cuda_drv.forward (a zero logit row appended, softmax over dim 1, 'bsdh,bshw->bdhw':
+ * example-setfind/setfind.py:128-136, python/l1attn_sparse.py:488-506) and the form its README asks
+ * for (README.md:21).  q,k [B,T,H,W]; v,vo [B,T,H,Wv].  Forward only.  Deterministic.
+ * f32: W == Wv in {16,32,64}, T >= 32 and 16-byte aligned pointers run the tiled kernel; every other
+ * shape, and f64, a generic one (L1ATTN_ERR_RANGE when it would need 2^32 threads or more).
+ */
+int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse,
+                         int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
+int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, double* vo, double* lse,
+                         int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
+
 /* -------------------------------------------------------------------------- edge lists */
 
 /*

@@ -54,6 +54,10 @@ def lib():
             f.restype = ctypes.c_int
             f.argtypes = [_c_p] * 5 + [_c_i64] * 4 + [_c_p, _c_sz, _c_p]
         _c_i = ctypes.c_int
+        for sfx in ("f32", "f64"):
+            f = getattr(L, "l1attn_fused_fwd_" + sfx)
+            f.restype = _c_i
+            f.argtypes = [_c_p] * 5 + [_c_i64] * 5 + [_c_p]
         L.l1attn_dense_column_ranks_f32.restype = _c_i
         L.l1attn_dense_column_ranks_f32.argtypes = [_c_p] * 4 + [_c_i64] * 4 + [_c_p]
         L.l1attn_expand_coo_workspace_bytes.restype = _c_sz
@@ -180,6 +184,29 @@ def dense_backward(d_attn, q, k):
             ptr(ws) if ws is not None else None, ws_bytes, stream_of(q))
     check(rc, "l1attn_dense_bwd_" + sfx)
     return [dq, dk]
+
+
+def dense_fused_forward(q, k, v, want_lse=False):
+    """Fused forward: vo[b,t,h,:] = sum_s p[s] * v[b,s,h,:] with p the softmax over src of the L1 logits
+    and a no-op zero logit (1 + sum in the denominator), without materialising the [B,T,T,H] logits.
+    What example-setfind/setfind.py:128-136 composes from L1Attn, softmax and einsum.
+    Returns [vo, lse]; lse [B,T,H] = log(1 + sum_s exp(a)) if want_lse else None."""
+    for x, n in ((q, "q"), (k, "k"), (v, "v")):
+        check_input(x, n)
+    if q.dim() != 4 or q.shape != k.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
+        raise RuntimeError("q, k, v must be [batch, n_ctx, n_heads, width] tensors with equal leading dims")
+    if not (v.dtype == q.dtype == k.dtype) or not (v.device == q.device == k.device):
+        raise RuntimeError("q, k, v must share dtype and device")
+    B, T, H, W = q.shape
+    Wv = v.shape[3]
+    sfx = sfx_of(q)
+    vo = torch.empty_like(v)
+    lse = torch.empty((B, T, H), dtype=q.dtype, device=q.device) if want_lse else None
+    with torch.cuda.device(q.device):
+        rc = getattr(lib(), "l1attn_fused_fwd_" + sfx)(
+            ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse) if lse is not None else None, B, T, H, W, Wv, stream_of(q))
+    check(rc, "l1attn_fused_fwd_" + sfx)
+    return [vo, lse]
 
 
 # ------------------------------------------------------------------------------- edge lists

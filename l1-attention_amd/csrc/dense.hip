@@ -24,6 +24,7 @@
 // Generic kernels (any shape, float or double, exact comparisons) cover everything else.
 #include "common.h"
 #include "dense_rank.h"
+#include "xcd.h"
 #include <math.h>
 #include <algorithm>
 
@@ -138,24 +139,6 @@ __global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict_
 constexpr int FWD_SJ = 8;  // src rows finished between two output flushes
 constexpr int FWD_L2_AHEAD = 4;  // src blocks between the L2 prefetch of k rows and their use
 constexpr int FWD_TILE = 1024 + 4 * WAVE;  // floats per staged src row: 64*NW outputs + one pad column per sub-tile (NH >= 4)
-
-// Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.
-// This maps the flat dispatch index to a logical one such that logically consecutive workgroups
-// (which share k rows) land on the same XCD: XCD x runs the logical range [x*n/8, (x+1)*n/8).
-struct LogicalBlock { int x, y, z; };
-__device__ __forceinline__ LogicalBlock xcd_remap()
-{
-	const unsigned nx = gridDim.x, ny = gridDim.y, n = nx * ny * gridDim.z;
-	const unsigned flat = blockIdx.x + nx * (blockIdx.y + ny * blockIdx.z);
-	const unsigned per = n / 8u;
-	unsigned m = flat;
-	if (flat < per * 8u) m = (flat % 8u) * per + flat / 8u;
-	LogicalBlock lb;
-	lb.x = (int)(m % nx);
-	lb.y = (int)((m / nx) % ny);
-	lb.z = (int)(m / (nx * ny));
-	return lb;
-}
 
 // grid.x = dst tiles of 64*NTS tokens, grid.y = src chunks, grid.z = B * head groups.
 // block = 64 * NW threads (NW <= 16 waves) = NH heads x NTS dst sub-tiles of 64 tokens: wave w owns head
@@ -823,6 +806,7 @@ int launch_fwd_generic(const T* q, const T* k, T* attn, int64_t B, int64_t Tn, i
 		L1_LAUNCH_CHECK();
 		return L1ATTN_OK;
 	}
+	if (Tn * H >= ((int64_t)1 << 32)) return L1ATTN_ERR_RANGE;  // threads along x of one launch
 	dim3 grid((unsigned)l1_cdiv(Tn * H, 256), (unsigned)std::min<int64_t>(B * Tn, 65535), 1);
 	hipLaunchKernelGGL(dense_fwd_generic<T>, grid, dim3(256), 0, st, q, k, attn, B, Tn, H, W, scale);
 	L1_LAUNCH_CHECK();
@@ -835,6 +819,7 @@ int launch_bwd_generic(const T* dA, const T* q, const T* k, T* dq, T* dk, int64_
 {
 	const T scale = (T)(-1.0 / sqrt((double)W));
 	const int64_t n = B * Tn * H * W;
+	if (n >= ((int64_t)1 << 32)) return L1ATTN_ERR_RANGE;  // one thread per gradient element
 	dim3 grid((unsigned)l1_cdiv(n, 256));
 	hipLaunchKernelGGL(dense_bwd_generic_dq<T>, grid, dim3(256), 0, st, dA, q, k, dq, B, Tn, H, W, scale);
 	L1_LAUNCH_CHECK();

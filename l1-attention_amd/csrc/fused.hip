@@ -1,0 +1,176 @@
+// Fused dense L1 attention for gfx950, forward only: logits, softmax over the src tokens with the
+// "no-op" zero logit, and the value sum, without ever writing the [B,T,T,H] logits:
+//
+//   a[s]        = -1/sqrt(W) * sum_w |q[b,t,h,w] - k[b,s,h,w]|
+//   vo[b,t,h,:] = sum_s exp(a[s]) * v[b,s,h,:] / (1 + sum_s exp(a[s]))
+//
+// This is what the reference's model code computes from the dense operator (L1Attn, a row of zero
+// logits appended, softmax over dim 1, einsum 'bsdh,bshw->bdhw': example-setfind/setfind.py:128-136,
+// python/l1attn_sparse.py:488-506) and what its README names as the better form ("blocked attention
+// ... ala FlashAttention", README.md:21).  It also equals sparse attention over the full cartesian
+// edge list.  Every logit is <= 0 and the no-op logit is 0, so the softmax needs no running maximum:
+// exp(a) <= 1 and the denominator is >= 1.
+//
+// Tiled kernel: one wavefront per head, one lane per dst token, as in the dense forward.  A lane keeps
+// its q row (W registers) and its output row (WV registers); the k and v rows of the current src token
+// are wave-uniform and come through the scalar cache.  Per pair-element: v_sub, v_add |x| for the logit
+// and one v_fmac for the value sum; one exp per (src, dst, head).  No LDS, no atomics; src tokens are
+// summed in ascending order, so results repeat bit for bit.
+#include "common.h"
+#include "xcd.h"
+#include <math.h>
+
+namespace {
+
+template <typename T> __device__ __forceinline__ T fabs_t(T x) { return x < (T)0 ? -x : x; }
+template <typename T> __device__ __forceinline__ T exp_t(T x);
+template <> __device__ __forceinline__ float exp_t<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double exp_t<double>(double x) { return exp(x); }
+__device__ __forceinline__ float log_t(float x) { return logf(x); }
+__device__ __forceinline__ double log_t(double x) { return log(x); }
+
+// Any shape, float or double: one thread per output element (b,t,h,wv); the logit of each src token is
+// recomputed by every thread of the row (W-fold redundant), which only small or odd shapes pay.
+template <typename T>
+__global__ __launch_bounds__(256) void fused_fwd_generic(const T* __restrict__ q, const T* __restrict__ k,
+                                                           const T* __restrict__ v, T* __restrict__ vo,
+                                                           T* __restrict__ lse, int64_t B, int64_t Tn, int64_t H,
+                                                           int64_t W, int64_t Wv, T scale)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= B * Tn * H * Wv) return;
+	const int64_t wv = idx % Wv, h = (idx / Wv) % H, t = (idx / (Wv * H)) % Tn, b = idx / (Wv * H * Tn);
+	const T* qp = q + ((b * Tn + t) * H + h) * W;
+	T den = 0, acc = 0;
+	for (int64_t s = 0; s < Tn; s++) {
+		const T* kp = k + ((b * Tn + s) * H + h) * W;
+		T f = 0;
+		for (int64_t w = 0; w < W; w++) f += fabs_t(qp[w] - kp[w]);
+		const T p = exp_t(f * scale);
+		den += p;
+		acc += p * v[((b * Tn + s) * H + h) * Wv + wv];
+	}
+	den += (T)1;
+	vo[idx] = acc / den;
+	if (lse && wv == 0) lse[(b * Tn + t) * H + h] = log_t(den);
+}
+
+// grid.x = dst tiles of 64 tokens, grid.y = B * head groups; block = 64 * NH threads, wave w owns head
+// hg*NH + w.  W == WV is a compile-time multiple of 16; q, k, v, vo must be 16-byte aligned.
+template <int W>
+__global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restrict__ q, const float* __restrict__ k,
+                                                            const float* __restrict__ v, float* __restrict__ vo,
+                                                            float* __restrict__ lse, int Tn, int H, int n_hg, int NH,
+                                                            float scale)
+{
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.y / n_hg, hg = lb.y % n_hg;
+	const int h_raw = hg * NH + wave;
+	const int h = min(h_raw, H - 1);  // surplus waves of the last group redo head H-1 and store nothing
+	const int t_raw = lb.x * 64 + lane;
+	const int t = min(t_raw, Tn - 1);  // surplus lanes of the last tile redo token Tn-1 and store nothing
+	const bool store = h_raw < H && t_raw < Tn;
+
+	float qr[W], acc[W];
+	{
+		const float4* qp = reinterpret_cast<const float4*>(q + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = qp[w4];
+			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
+		}
+#pragma unroll
+		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+	}
+	float den = 0.0f;
+	const int64_t row = (int64_t)H * W;
+	const float* kp = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;  // src token 0 of this (b,h): wave-uniform
+	const float* vp = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	for (int s = 0; s < Tn; s++) {
+		float a = 0.0f;
+#pragma unroll
+		for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);  // uniform address: scalar loads
+		const float p = expf(a * scale);
+		den += p;
+#pragma unroll
+		for (int w = 0; w < W; w++) acc[w] += p * vp[w];
+		kp += row;
+		vp += row;
+	}
+	den += 1.0f;
+	if (store) {
+		const float inv = 1.0f / den;
+		float4* op = reinterpret_cast<float4*>(vo + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++)
+			op[w4] = make_float4(acc[w4 * 4 + 0] * inv, acc[w4 * 4 + 1] * inv, acc[w4 * 4 + 2] * inv,
+			                     acc[w4 * 4 + 3] * inv);
+		if (lse) lse[((int64_t)b * Tn + t) * H + h] = logf(den);
+	}
+}
+
+bool shape_ok(int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv)
+{
+	return B >= 0 && T >= 0 && H >= 0 && W >= 1 && Wv >= 1;
+}
+
+template <typename T>
+int launch_generic(const T* q, const T* k, const T* v, T* vo, T* lse, int64_t B, int64_t Tn, int64_t H, int64_t W,
+                   int64_t Wv, hipStream_t st)
+{
+	const int64_t n = B * Tn * H * Wv;
+	if (n >= ((int64_t)1 << 32)) return L1ATTN_ERR_RANGE;  // one thread per output element
+	const T scale = (T)(-1.0 / sqrt((double)W));
+	hipLaunchKernelGGL(fused_fwd_generic<T>, dim3((unsigned)l1_cdiv(n, 256)), dim3(256), 0, st, q, k, v, vo, lse, B, Tn,
+	                   H, W, Wv, scale);
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse, int64_t B, int64_t T,
+                         int64_t H, int64_t W, int64_t Wv, void* stream)
+{
+	if (!shape_ok(B, T, H, W, Wv)) return L1ATTN_ERR_ARG;
+	if (B * T * H == 0) return L1ATTN_OK;
+	if (!q || !k || !v || !vo) return L1ATTN_ERR_ARG;
+	hipStream_t st = (hipStream_t)stream;
+	const bool aligned = ((((uintptr_t)q) | ((uintptr_t)k) | ((uintptr_t)v) | ((uintptr_t)vo)) & 15) == 0;
+	const int NH = (int)(H < 4 ? H : 4);
+	const int64_t n_hg = l1_cdiv(H, NH);
+	const bool tiled = aligned && W == Wv && (W == 16 || W == 32 || W == 64) && T >= 32 && T <= (1 << 30) &&
+	                   B * n_hg <= 65535 && H <= 65535;
+	if (!tiled) return launch_generic<float>(q, k, v, vo, lse, B, T, H, W, Wv, st);
+	const float scale = (float)(-1.0 / sqrt((double)W));
+	const dim3 grid((unsigned)l1_cdiv(T, 64), (unsigned)(B * n_hg), 1), block(64 * NH);
+#define L1_FUSED_CASE(WV)                                                                                        \
+	case WV:                                                                                                     \
+		hipLaunchKernelGGL(fused_fwd_f32_tile<WV>, grid, block, 0, st, q, k, v, vo, lse, (int)T, (int)H, (int)n_hg, \
+		                   NH, scale);                                                                           \
+		break
+	switch (W) {
+		L1_FUSED_CASE(16);
+		L1_FUSED_CASE(32);
+		L1_FUSED_CASE(64);
+	default: return L1ATTN_ERR_ARG;
+	}
+#undef L1_FUSED_CASE
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, double* vo, double* lse, int64_t B,
+                         int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream)
+{
+	if (!shape_ok(B, T, H, W, Wv)) return L1ATTN_ERR_ARG;
+	if (B * T * H == 0) return L1ATTN_OK;
+	if (!q || !k || !v || !vo) return L1ATTN_ERR_ARG;
+	return launch_generic<double>(q, k, v, vo, lse, B, T, H, W, Wv, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -39,3 +39,26 @@ class L1Attn(nn.Module):
 
     def forward(self, q, k):
         return L1AttnFn.apply(q, k)
+
+
+class L1AttnFusedFn(Function):
+    """L1 attention with the value sum fused in (forward only): softmax over the src tokens of the L1
+    logits with the no-op zero logit, times v, without the [B,T,T,H] tensor.  Equals
+    einsum('bsdh,bshw->bdhw', softmax(cat(L1Attn()(q,k), zeros), 1)[:, :-1], v), the composition of
+    example-setfind/setfind.py:128-136.  The reference has no such function (README.md:21 asks for it)."""
+    @staticmethod
+    def forward(ctx, q, k, v):
+        vo, _ = _drv.dense_fused_forward(q.contiguous(), k.contiguous(), v.contiguous())
+        return vo
+
+    @staticmethod
+    def backward(ctx, d_vo):
+        raise RuntimeError("L1AttnFused has no backward: use L1Attn with softmax and einsum for training")
+
+
+class L1AttnFused(nn.Module):
+    def __init__(self):
+        super(L1AttnFused, self).__init__()
+
+    def forward(self, q, k, v):
+        return L1AttnFusedFn.apply(q, k, v)

@@ -82,6 +82,19 @@ def dense_bwd(d_attn, q, k):
     return dq, dk
 
 
+def fused_fwd(q, k, v):
+    """The composition the reference's model code builds on the dense operator
+    (example-setfind/setfind.py:128-136; python/l1attn_sparse.py:488-506, testsparse.py:50-62):
+    logits from dense_fwd (cpp/l1attn_drv.cpp:13-55), a row of zero logits appended along src,
+    softmax over src, the no-op row dropped, einsum 'bsdh,bshw->bdhw' with v.
+    -> (vo [B,T,H,Wv], lse [B,T,H] = log of the softmax denominator)."""
+    B, T, H, W = q.shape
+    a = dense_fwd(q, k)
+    a = torch.cat((a, torch.zeros(B, 1, T, H, dtype=a.dtype)), 1)
+    p = torch.softmax(a, 1)[:, :T]
+    return torch.einsum("bsdh,bshw->bdhw", p, v), torch.logsumexp(a, 1)
+
+
 def _coo32(coo):
     coo = coo.to(torch.int32).contiguous()
     assert coo.dim() == 2 and coo.shape[1] >= 3

@@ -303,6 +303,13 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
         drv.dense_backward(torch.zeros(B, T, T, H + 1), q, k)
     with pytest.raises(RuntimeError, match="one shape"):
         drv.dense_backward(torch.zeros(B, T, T, H), q, torch.zeros(B, T, H, W + 1))
+    vo, lse = drv.dense_fused_forward(q, k, v, want_lse=True)
+    assert vo.shape == v.shape and lse.shape == (B, T, H) and _FakeLib.calls[-1] == "l1attn_fused_fwd_f32"
+    assert drv.dense_fused_forward(q.double(), k.double(), v.double())[1] is None
+    with pytest.raises(RuntimeError, match="equal leading dims"):
+        drv.dense_fused_forward(q, k, torch.zeros(B, T + 1, H, Wv))
+    with pytest.raises(RuntimeError, match="share dtype"):
+        drv.dense_fused_forward(q, k, v.double())
     plan = drv.plan_for(coo, T)
     assert (plan.E, plan.T, plan.max_dst_deg, plan.max_src_deg) == (E, T, 3, 2)
     assert drv.plan_for(coo, T) is plan                      # cached on the tensor
@@ -375,3 +382,9 @@ def test_operator_modules_autograd_plumbing_without_a_gpu(monkeypatch):
     vo = l1attn_sparse_bidi_cuda.L1AttnSparseBidi()(vf, vb, q, k, coo, 2, True)
     vo.sum().backward()
     assert all(t.grad is not None and t.grad.shape == t.shape for t in (vf, vb, q, k))
+    # the fused forward has no backward and says so
+    q, k, v = mk(B, T, H, W), mk(B, T, H, W), mk(B, T, H, W)
+    vo = l1attn_cuda.L1AttnFused()(q, k, v)
+    assert vo.shape == v.shape
+    with pytest.raises(RuntimeError, match="no backward"):
+        vo.sum().backward()

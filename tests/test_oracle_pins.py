@@ -223,6 +223,31 @@ def test_sparse_full_list_equals_dense_with_noop(sm):
         assert torch.allclose(vo2, expect, rtol=1e-13, atol=1e-13)
 
 
+def test_fused_forward_oracle_pins():
+    """oracle.fused_fwd (dense logits, no-op row, softmax over src, value sum) against three statements
+    that share no code with it: the sparse oracle over the full cartesian list (itself pinned by the
+    reference extension's golden vectors), the broadcast closed form, and a hand answer on the integer
+    fixture (python/l1attn_sparse.py:450-470; W = 3)."""
+    for q, k, v in (integer_fixture(), onehot_fixture()):
+        T = q.shape[1]
+        vo, lse = oracle.fused_fwd(q, k, v)
+        coo, dmx, _ = oracle.expand_coo(torch.cartesian_prod(torch.arange(T), torch.arange(T)))
+        ref, _ = oracle.sparse_fwd(v, q, k, coo, dmx, True)
+        assert torch.allclose(vo, ref, rtol=1e-13, atol=1e-13)
+        assert torch.allclose(vo, cf.dense_then_value(q, k, v, noop=True), rtol=1e-13, atol=1e-13)
+        den = 1.0 + cf.dense_attn(q, k).exp().sum(1)
+        assert torch.allclose(lse, den.log(), rtol=1e-13, atol=1e-13)
+    # a transposed src/dst or a dropped "+1" must fail: asymmetric random case, denominators near 1
+    g = torch.Generator().manual_seed(12)
+    q, k, v = (torch.randn(2, 5, 3, 4, generator=g, dtype=torch.float64) for _ in range(3))
+    vo, lse = oracle.fused_fwd(q, k, v)
+    for b, t, h in ((0, 0, 0), (1, 4, 2), (0, 3, 1)):
+        e = [math.exp(-float((q[b, t, h] - k[b, s, h]).abs().sum()) / 2.0) for s in range(5)]  # sqrt(4) = 2
+        expect = sum(e[s] * v[b, s, h] for s in range(5)) / (1.0 + sum(e))
+        assert torch.allclose(vo[b, t, h], expect, rtol=1e-13, atol=1e-15)
+        assert abs(float(lse[b, t, h]) - math.log(1.0 + sum(e))) < 1e-13
+
+
 def test_sparse_integer_fixture_hand_answer():
     # python/l1attn_sparse.py:484 : co = [[0,0],[0,1],[1,0],[1,1],[2,2]], softmax on.
     # dst 0 sees k0 (L1=4) and k1 (L1=0): e = exp(-4/sqrt3), 1 ; denominator 1 + e + 1.

@@ -1,0 +1,115 @@
+"""GPU parity of the fused forward (L1 logits, softmax over src with the no-op logit, value sum in one
+kernel) through l1attn_cuda.L1AttnFused and so through l1attn_fused_fwd_{f32,f64}.
+
+This file has not run on a GPU yet, which is why its name keeps it out of pytest's collection
+(run it as `python -m pytest tests/wip_fused_gpu.py -m gpu`); rename it to test_*.py once it has
+passed there.
+
+Yardsticks: the CPU oracle (oracle.fused_fwd: the reference's dense CPU loop, then the no-op row,
+softmax and einsum of example-setfind/setfind.py:128-136) at small sizes; at sizes the oracle's
+[B,T,T,H] tensor would be slow for, the same composition in fp64 on the device from the dense HIP
+operator (itself checked against the oracle elsewhere).  Tolerances: fp32 max|x-ref|/max|ref| <= 1e-5
+against fp64 on the same fp32-valued inputs; fp64 entry point <= 1e-12.
+"""
+import pytest
+import torch
+
+import closed_forms as cf
+import workloads
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL, F64_TOL = 1e-5, 1e-12
+
+
+def _fused():
+    import l1attn_cuda
+    return l1attn_cuda
+
+
+SHAPES = [
+    # B, T, H, W, Wv
+    (2, 64, 4, 32, 32),     # first baseline configuration: tiled kernel, width 32
+    (1, 100, 3, 64, 64),    # tiled kernel, ragged last dst tile, fewer heads than a workgroup holds
+    (2, 70, 6, 16, 16),     # tiled kernel, width 16, ragged head group (6 = 4 + 2)
+    (1, 33, 9, 64, 64),     # three head groups, the last with one head
+    (2, 3, 16, 7, 7),       # generic kernel (check_sparse.py:18-21 shape)
+    (1, 40, 2, 48, 48),     # generic kernel: width not among the tiled ones
+    (1, 37, 3, 32, 20),     # generic kernel: value width differs
+    (1, 31, 2, 64, 64),     # generic kernel: fewer than 32 tokens
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fused_forward_vs_oracle(shape):
+    B, T, H, W, Wv = shape
+    print("case fused", shape, flush=True)
+    import _l1attn_hip as drv
+    g = torch.Generator().manual_seed(sum(shape))
+    q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))
+    v = torch.randn(B, T, H, Wv, generator=g)
+    if W == Wv:
+        ref, ref_lse = oracle.fused_fwd(q.double(), k.double(), v.double())
+    else:
+        ref = cf.dense_then_value(q.double(), k.double(), v.double(), noop=True)
+        ref_lse = (1.0 + cf.dense_attn(q.double(), k.double()).exp().sum(1)).log()
+    vo, lse = drv.dense_fused_forward(q.cuda(), k.cuda(), v.cuda(), want_lse=True)
+    torch.cuda.synchronize()
+    assert cf.rel_err(vo.cpu(), ref) <= F32_TOL
+    assert cf.rel_err(lse.cpu(), ref_lse) <= F32_TOL
+    vo2 = _fused().L1AttnFused()(q.cuda(), k.cuda(), v.cuda())
+    assert torch.equal(vo2, vo)  # module == driver, and bitwise run-to-run
+    vo64, lse64 = drv.dense_fused_forward(q.double().cuda(), k.double().cuda(), v.double().cuda(), want_lse=True)
+    assert cf.rel_err(vo64.cpu(), ref) <= F64_TOL
+    assert cf.rel_err(lse64.cpu(), ref_lse) <= F64_TOL
+
+
+def test_fused_forward_unaligned_views_take_the_generic_kernel():
+    print("case fused unaligned", flush=True)
+    import _l1attn_hip as drv
+    g = torch.Generator().manual_seed(3)
+    B, T, H, W = 1, 64, 2, 32
+    flat = torch.randn(3, B * T * H * W + 1, generator=g).cuda()
+    q, k, v = (flat[i, 1:].view(B, T, H, W) for i in range(3))  # 4-byte aligned only
+    assert q.data_ptr() % 16 != 0 and q.is_contiguous()
+    vo, _ = drv.dense_fused_forward(q, k, v)
+    ref, _ = oracle.fused_fwd(q.cpu().double(), k.cpu().double(), v.cpu().double())
+    assert cf.rel_err(vo.cpu(), ref) <= F32_TOL
+
+
+@pytest.mark.parametrize("layernorm", [False, True])
+def test_fused_forward_second_baseline_shape_vs_dense_operator(layernorm):
+    """B16 T1024 H8 W64 (second baseline configuration, with its downstream softmax and einsum) at B=2:
+    the fused kernel against the same composition in fp64 built on the dense HIP operator's fp64 entry."""
+    print("case fused config 2", layernorm, flush=True)
+    fz = _fused()
+    B, T, H, W = 2, 1024, 8, 64
+    q, k, v = workloads.dense_inputs(B, T, H, W, seed=1002, layernorm=layernorm, with_v=True)
+    q, k, v = q.cuda(), k.cuda(), v.cuda()
+    vo = fz.L1AttnFused()(q, k, v)
+    a = fz.L1Attn()(q.double(), k.double())
+    a = torch.cat((a, torch.zeros(B, 1, T, H, dtype=a.dtype, device=a.device)), 1)
+    ref = torch.einsum("bsdh,bshw->bdhw", torch.softmax(a, 1)[:, :T], v.double())
+    assert cf.rel_err(vo.cpu(), ref.cpu()) <= F32_TOL
+    # equals sparse attention over the full cartesian list (python/l1attn_sparse.py:488-506)
+    import l1attn_sparse_cuda as sp
+    Ts = 96
+    co = torch.cartesian_prod(torch.arange(Ts), torch.arange(Ts)).cuda()
+    coo, dmx, _ = sp.expandCoo(co, warn=False)
+    qs, ks, vs = (x[:, :Ts].contiguous() for x in (q, k, v))
+    assert cf.rel_err(fz.L1AttnFused()(qs, ks, vs).cpu(), sp.L1AttnSparse()(vs, qs, ks, coo, dmx).cpu().double()) <= 2e-5
+
+
+def test_fused_forward_no_backward_and_input_checks():
+    print("case fused checks", flush=True)
+    fz = _fused()
+    import _l1attn_hip as drv
+    x = torch.randn(1, 32, 2, 16).cuda().requires_grad_()
+    vo = fz.L1AttnFused()(x, x, x)
+    with pytest.raises(RuntimeError, match="no backward"):
+        vo.sum().backward()
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        drv.dense_fused_forward(x.detach().cpu(), x.detach(), x.detach())
+    with pytest.raises(RuntimeError, match="only float32 and float64"):
+        drv.dense_fused_forward(x.detach().half(), x.detach().half(), x.detach().half())
