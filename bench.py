@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the L1-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-sparse] [--skip-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-sparse] [--skip-cpu] [--extra]
 
 A step is one dense L1Attn forward + backward (through the reference's Python API,
 l1attn_cuda.L1AttnFn) over the headline configuration  q,k fp32 [B=8, T=4096, H=16, W=64],
@@ -167,6 +167,56 @@ def sparse_configs(skip_cpu):
     return res
 
 
+def extra_legs():
+    """Opt-in (--extra): the two additions beyond the reference's operators, timed beside what they replace.
+    Fused forward (logits, softmax over src with the no-op logit, value sum in one kernel) against the same
+    result composed from L1Attn and torch's cat / softmax / einsum, at the second baseline configuration and
+    the headline shape; sparse and bidirectional forwards with float16 / bfloat16 rows against float32 rows at
+    configurations 4 and 5.  Prints its own JSON line; the default run does not come here."""
+    import torch
+    import workloads
+    import l1attn_cuda
+    import l1attn_sparse_cuda as sp
+    import l1attn_sparse_bidi_cuda as bi
+    dev = torch.device("cuda:0")
+    res = {"fused_forward": {}, "sparse_forward_16bit": {}}
+    for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
+        q, k, v = (x.to(dev) for x in workloads.dense_inputs(B, T, H, W, seed=1002, with_v=True))
+        fused, plain = l1attn_cuda.L1AttnFused(), l1attn_cuda.L1Attn()
+
+        def composed():
+            a = plain(q, k)
+            a = torch.cat((a, torch.zeros(B, 1, T, H, device=dev)), 1)
+            return torch.einsum("bsdh,bshw->bdhw", torch.softmax(a, 1)[:, :T], v)
+
+        ms_f = time_gpu(lambda: fused(q, k, v), 5)
+        big = B * T * T * H * 4 > (4 << 30)  # the composition holds three [B,T,T,H] tensors at once
+        ms_c = time_gpu(composed, 2 if big else 5, warm=1)
+        err = float((fused(q, k, v) - composed()).abs().max() / composed().abs().max())
+        N = B * T * T * H * W
+        res["fused_forward"][name] = {
+            "fused_ms": ms_f, "composed_ms": ms_c, "speedup": ms_c / ms_f, "max_rel_diff": err,
+            "fused_tops": 3 * N / ms_f / 1e9, "frac_of_valu_peak": 3 * N / ms_f / 1e9 / P_VALU_TOPS,
+            "note": "3 algorithmic ops per pair-element (sub, abs-accumulate, multiply-accumulate)"}
+        log(name, json.dumps(res["fused_forward"][name]))
+        del q, k, v
+        torch.cuda.empty_cache()
+    for name, bidi, (B, T, H, W), co in (
+            ("config4_uni", False, (4, 4096, 8, 32), workloads.uniform_degree_graph(4096, 64, seed=1004)),
+            ("config5_bidi", True, (1, 65536, 4, 64), workloads.powerlaw_graph(65536, seed=1005))):
+        coo, dmx, smx = sp.expandCoo(co.to(dev), warn=False)
+        x32 = [t.to(dev) for t in workloads.sparse_inputs(B, T, H, W, seed=1004 + bidi, n=4)]
+        m = bi.L1AttnSparseBidi() if bidi else sp.L1AttnSparse()
+        row = {"edges": int(co.shape[0])}
+        for dt in (torch.float32, torch.float16, torch.bfloat16):
+            x = [t.to(dt) for t in x32]
+            args = (x[0], x[1], x[2], x[3]) if bidi else (x[0], x[2], x[3])
+            row[str(dt).split(".")[1] + "_fwd_ms"] = time_gpu(lambda: m(*args, coo, dmx), 10)
+        res["sparse_forward_16bit"][name] = row
+        log(name, json.dumps(row))
+    return res
+
+
 def valu_probe():
     """What ordinary (non-packed) fp32 VALU code sustains on this GPU: the library's register-only probe on
     256 workgroups of 8 waves (two waves per SIMD on every CU), HIP events on the current stream."""
@@ -246,6 +296,8 @@ def main():
     ap.add_argument("--skip-sparse", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-dense", action="store_true", help="profiling aid: sparse legs only")
+    ap.add_argument("--extra", action="store_true",
+                    help="only time the fused forward and the 16-bit sparse forwards beside what they replace")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: only run three 1 GiB device-to-device copies, the known-size "
                          "kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -272,6 +324,9 @@ def main():
         return
     if args.skip_dense:
         print(json.dumps({"sparse": sparse_configs(True)}), flush=True)
+        return
+    if args.extra:
+        print(json.dumps({"extra": extra_legs()}), flush=True)
         return
 
     log("dense headline ...")
