@@ -214,7 +214,35 @@ def extra_legs():
             row[str(dt).split(".")[1] + "_fwd_ms"] = time_gpu(lambda: m(*args, coo, dmx), 10)
         res["sparse_forward_16bit"][name] = row
         log(name, json.dumps(row))
+    res["instruction_rates"] = instruction_rates()
     return res
+
+
+def instruction_rates():
+    """Issue rates of candidate instructions from the library's register-only probe (256 workgroups of 8 waves),
+    in wave-instructions per SIMD and nanosecond and as lane-operations per second."""
+    import torch
+    import _l1attn_hip as drv
+    L = drv.lib()
+    blocks, iters = 256, 4000
+    out = torch.empty(blocks * 512, dtype=torch.float32, device="cuda:0")
+    st = drv.stream_of(out)
+    names = {0: "v_fmac_f32", 1: "v_sad_u32 (VGPR operands)", 2: "v_sad_u32 (SGPR operand)",
+             3: "v_sub_f32 + v_add_f32 |x| (two instructions per step)"}
+    rates = {}
+    for op, name in names.items():
+        assert L.l1attn_probe_valu_op(drv.ptr(out), blocks, 100, op, st) == 0
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record()
+        assert L.l1attn_probe_valu_op(drv.ptr(out), blocks, iters, op, st) == 0
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1])
+        steps = blocks * 8 * iters * 64
+        rates[name] = {"ms": ms, "steps_per_simd_ns": steps / (256 * 4) / (ms * 1e6),
+                       "lane_steps_tops": steps * 64 / (ms * 1e-3) / 1e12}
+    return rates
 
 
 def valu_probe():

@@ -41,6 +41,13 @@ int l1attn_version(void);
  * one instruction per SIMD every two cycles.  out: blocks*512 floats.  Asynchronous.
  */
 int l1attn_probe_valu(float* out, int64_t blocks, int64_t iters, void* stream);
+/*
+ * The same probe for other instructions (same geometry and accounting), to learn an instruction's
+ * issue rate before a kernel is built on it: op 0 = v_fmac_f32 (as above), 1 = v_sad_u32 (|a-b|+c on
+ * unsigned integers in one instruction) on VGPRs, 2 = v_sad_u32 with an SGPR operand, 3 = pairs of
+ * v_sub_f32 and v_add_f32 |x| (2 instructions per counted step).  No counterpart in the reference.
+ */
+int l1attn_probe_valu_op(float* out, int64_t blocks, int64_t iters, int op, void* stream);
 
 /* ------------------------------------------------------------------------------ dense */
 

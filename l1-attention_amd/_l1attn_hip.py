@@ -38,6 +38,8 @@ def lib():
         L.l1attn_version.restype = ctypes.c_int
         L.l1attn_probe_valu.restype = ctypes.c_int
         L.l1attn_probe_valu.argtypes = [_c_p, _c_i64, _c_i64, _c_p]
+        L.l1attn_probe_valu_op.restype = ctypes.c_int
+        L.l1attn_probe_valu_op.argtypes = [_c_p, _c_i64, _c_i64, ctypes.c_int, _c_p]
         L.l1attn_dense_fwd_workspace_bytes.restype = _c_sz
         L.l1attn_dense_fwd_workspace_bytes.argtypes = [_c_i64] * 4
         L.l1attn_dense_fwd_ws_f32.restype = ctypes.c_int

@@ -113,3 +113,15 @@ def test_fused_forward_no_backward_and_input_checks():
         drv.dense_fused_forward(x.detach().cpu(), x.detach(), x.detach())
     with pytest.raises(RuntimeError, match="only float32 and float64"):
         drv.dense_fused_forward(x.detach().half(), x.detach().half(), x.detach().half())
+
+
+def test_probe_other_instructions_runs():
+    """The instruction-rate probe launches for every op code and rejects an unknown one."""
+    print("case probe ops", flush=True)
+    import _l1attn_hip as drv
+    L = drv.lib()
+    out = torch.zeros(4 * 512, device="cuda")
+    for op in range(4):
+        assert L.l1attn_probe_valu_op(drv.ptr(out), 4, 3, op, drv.stream_of(out)) == 0
+    torch.cuda.synchronize()
+    assert L.l1attn_probe_valu_op(drv.ptr(out), 4, 3, 4, drv.stream_of(out)) == -1
