@@ -214,6 +214,23 @@ def extra_legs():
             row[str(dt).split(".")[1] + "_fwd_ms"] = time_gpu(lambda: m(*args, coo, dmx), 10)
         res["sparse_forward_16bit"][name] = row
         log(name, json.dumps(row))
+    import _l1attn_hip as drv
+    res["fixed_point_forward"] = {}
+    for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
+        q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
+        q, k = q.to(dev), k.to(dev)
+        ms32 = time_gpu(lambda: drv.dense_forward(q, k), 5)
+        msfx = time_gpu(lambda: drv.dense_forward_fixed(q, k), 5)
+        a32, afx = drv.dense_forward(q, k)[0], drv.dense_forward_fixed(q, k)[0]
+        diff = float((a32[0] - afx[0]).abs().max() / a32[0].abs().max())
+        N = B * T * T * H * W
+        res["fixed_point_forward"][name] = {
+            "fp32_ms": ms32, "fixed_ms": msfx, "fixed_tops_algorithmic": 2 * N / msfx / 1e9,
+            "max_rel_diff_to_fp32_kernel_batch0": diff,
+            "note": "fixed_ms includes the two conversion pre-passes and the workspace allocation"}
+        log(name, json.dumps(res["fixed_point_forward"][name]))
+        del q, k, a32, afx
+        torch.cuda.empty_cache()
     res["instruction_rates"] = instruction_rates()
     return res
 

@@ -44,6 +44,10 @@ def lib():
         L.l1attn_dense_fwd_workspace_bytes.argtypes = [_c_i64] * 4
         L.l1attn_dense_fwd_ws_f32.restype = ctypes.c_int
         L.l1attn_dense_fwd_ws_f32.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]
+        L.l1attn_dense_fwd_fixed_workspace_bytes.restype = _c_sz
+        L.l1attn_dense_fwd_fixed_workspace_bytes.argtypes = [_c_i64] * 4
+        L.l1attn_dense_fwd_fixed_f32.restype = ctypes.c_int
+        L.l1attn_dense_fwd_fixed_f32.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_p, _c_sz, _c_p]
         L.l1attn_dense_bwd_workspace_bytes.restype = _c_sz
         L.l1attn_dense_bwd_workspace_bytes.argtypes = [_c_i64] * 4
         L.l1attn_dense_bwd_plan_info.restype = ctypes.c_int
@@ -161,6 +165,25 @@ def dense_forward(q, k):
         else:
             rc = getattr(L, "l1attn_dense_fwd_" + sfx)(ptr(q), ptr(k), ptr(attn), B, T, H, W, stream_of(q))
     check(rc, "l1attn_dense_fwd_" + sfx)
+    return [attn]
+
+
+def dense_forward_fixed(q, k):
+    """Experimental float32 forward on fixed point (one v_sad_u32 per pair-element; inputs rounded to a
+    per-head grid of 2^-24 of the head's largest magnitude).  Same contract as dense_forward; widths 32 and
+    64 only.  Not used by L1AttnFn."""
+    check_input(q, "q")
+    check_input(k, "k")
+    if q.dim() != 4 or q.shape != k.shape or q.dtype != torch.float32 or k.dtype != torch.float32 or q.device != k.device:
+        raise RuntimeError("q and k must be float32 [batch, n_ctx, n_heads, width] tensors of one shape and device")
+    B, T, H, W = q.shape
+    attn = torch.empty((B, T, T, H), dtype=q.dtype, device=q.device)
+    L = lib()
+    with torch.cuda.device(q.device):
+        ws_bytes = L.l1attn_dense_fwd_fixed_workspace_bytes(B, T, H, W)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
+        rc = L.l1attn_dense_fwd_fixed_f32(ptr(q), ptr(k), ptr(attn), B, T, H, W, ptr(ws), ws_bytes, stream_of(q))
+    check(rc, "l1attn_dense_fwd_fixed_f32")
     return [attn]
 
 

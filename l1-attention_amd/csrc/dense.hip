@@ -223,10 +223,31 @@ __device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
 	asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(lo), "+s"(hi));
 }
 
-template <int W>
+// FIXED: q and k hold biased fixed-point values (32-bit unsigned, see fixed_quantise) on a grid of gq[b*H+h]
+// per (batch, head); the pair-element is then one v_sad_u32 (|a - b| + c on unsigned integers) instead of
+// v_sub + v_add |x|, the sum of W <= 64 terms is exact and at most 2^31, and the logit is sum * grid * scale.
+// Eight fixed-point pair-elements of the chunk at qv[0..8) / kv[i0..i0+8) in one volatile asm block: volatile
+// keeps it between the chunk's scalar prefetch and the next chunk's wait (both volatile asm), and one block per
+// eight instructions keeps the compiler from padding every inline instruction with a wait state.
+__device__ __forceinline__ void sad8(unsigned& au, const float* qv, const f32x16& kv, int i0)
+{
+#define L1_QU(i) "v"(__float_as_uint(qv[i]))
+#define L1_KU(i) "s"(__float_as_uint(kv[i0 + i]))  // (a bit_cast of a vector element reads element 0)
+	asm volatile("v_sad_u32 %0, %1, %9, %0\n\tv_sad_u32 %0, %2, %10, %0\n\tv_sad_u32 %0, %3, %11, %0\n\t"
+	             "v_sad_u32 %0, %4, %12, %0\n\tv_sad_u32 %0, %5, %13, %0\n\tv_sad_u32 %0, %6, %14, %0\n\t"
+	             "v_sad_u32 %0, %7, %15, %0\n\tv_sad_u32 %0, %8, %16, %0"
+	             : "+v"(au)
+	             : L1_QU(0), L1_QU(1), L1_QU(2), L1_QU(3), L1_QU(4), L1_QU(5), L1_QU(6), L1_QU(7),
+	               L1_KU(0), L1_KU(1), L1_KU(2), L1_KU(3), L1_KU(4), L1_KU(5), L1_KU(6), L1_KU(7));
+#undef L1_QU
+#undef L1_KU
+}
+
+template <int W, bool FIXED = false>
 __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restrict__ q, const float* __restrict__ k,
                                                              float* __restrict__ attn, int Tn, int H, int n_hg,
-                                                             int NH, int s_chunk, float scale, int V)
+                                                             int NH, int s_chunk, float scale, int V,
+                                                             const float* __restrict__ gq = nullptr)
 {
 	// V > 1: q and k rows of width V*W are read as V consecutive heads of width W (the same memory), so
 	// H counts those part-heads, NH (a multiple of V) of them share a workgroup, and the flush adds the V
@@ -268,6 +289,7 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 	// of the tensor (computed but never stored) read valid memory
 	const float* const k_last = kb + (int64_t)(Tn - 1) * krow + (CPR - 1) * 32;
 
+	if constexpr (FIXED) scale *= gq[b * (H / V) + h / V];  // wave-uniform
 	const int s_begin = lb.y * s_chunk;
 	const int s_end = min(Tn, s_begin + s_chunk);
 	f32x16 b0l, b0h, b1l, b1h;
@@ -280,6 +302,7 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 		// it is taken before the flush, by which time it has long arrived.
 		const float pf = kb[(int64_t)min(s0 + FWD_L2_AHEAD * FWD_SJ + (lane >> 3), Tn - 1) * krow + (lane & 7) * (W / 8)];
 		float a = 0.0f;
+		unsigned au = 0u;
 #pragma unroll
 		for (int c = 0; c < NCH; c++) {
 			const int j = c / CPR, part = c % CPR;
@@ -290,23 +313,37 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_pipe(const float* __restri
 				__builtin_amdgcn_sched_barrier(0);
 				sload32(b1l, b1h, kp);
 				__builtin_amdgcn_sched_barrier(0);
-				if (part == 0) a = 0.0f;
+				if (part == 0) { a = 0.0f; au = 0u; }
+				if constexpr (FIXED) {
+					sad8(au, &qr[part * 32], b0l, 0);
+					sad8(au, &qr[part * 32 + 8], b0l, 8);
+					sad8(au, &qr[part * 32 + 16], b0h, 0);
+					sad8(au, &qr[part * 32 + 24], b0h, 8);
+				} else {
 #pragma unroll
-				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + i] - b0l[i]);
+					for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + i] - b0l[i]);
 #pragma unroll
-				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b0h[i]);
+					for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b0h[i]);
+				}
 			} else {
 				swait32(b1l, b1h);
 				__builtin_amdgcn_sched_barrier(0);
 				sload32(b0l, b0h, kp);
 				__builtin_amdgcn_sched_barrier(0);
-				if (part == 0) a = 0.0f;
+				if (part == 0) { a = 0.0f; au = 0u; }
+				if constexpr (FIXED) {
+					sad8(au, &qr[part * 32], b1l, 0);
+					sad8(au, &qr[part * 32 + 8], b1l, 8);
+					sad8(au, &qr[part * 32 + 16], b1h, 0);
+					sad8(au, &qr[part * 32 + 24], b1h, 8);
+				} else {
 #pragma unroll
-				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + i] - b1l[i]);
+					for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + i] - b1l[i]);
 #pragma unroll
-				for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b1h[i]);
+					for (int i = 0; i < 16; i++) a += fabsf(qr[part * 32 + 16 + i] - b1h[i]);
+				}
 			}
-			if (part == CPR - 1) tile[j][(ts * WAVE + lane) * PH + hl] = a * scale;
+			if (part == CPR - 1) tile[j][(ts * WAVE + lane) * PH + hl] = FIXED ? (float)au * scale : a * scale;
 		}
 		asm volatile("" ::"v"(pf));
 		lds_barrier();
@@ -786,6 +823,44 @@ __global__ __launch_bounds__(256) void dense_pad_rows(const float* __restrict__ 
 	}
 }
 
+// Fixed-point forward, pre-pass 1: grid of each (batch, head) = largest |q| or |k| of the head * 2^-24
+// (at least the smallest normal float), so that every value is an integer of at most 2^24 in magnitude on it.
+// One workgroup per (b,h); the maximum is exact and order-independent.
+__global__ __launch_bounds__(256) void fixed_absmax(const float* __restrict__ q, const float* __restrict__ k,
+                                                      float* __restrict__ gq, int Tn, int H, int W)
+{
+	__shared__ float red[256];
+	const int b = blockIdx.x / H, h = blockIdx.x % H;
+	float m = 0.0f;
+	for (int i = threadIdx.x; i < Tn * W; i += 256) {
+		const int t = i / W, w = i - t * W;
+		const int64_t off = (((int64_t)b * Tn + t) * H + h) * (int64_t)W + w;
+		m = fmaxf(m, fmaxf(fabsf(q[off]), fabsf(k[off])));
+	}
+	red[threadIdx.x] = m;
+	__syncthreads();
+	for (int st = 128; st > 0; st >>= 1) {
+		if ((int)threadIdx.x < st) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + st]);
+		__syncthreads();
+	}
+	// 2^-24 of the maximum, but never below the smallest normal float (an all-zero or denormal-only head)
+	if (threadIdx.x == 0) gq[blockIdx.x] = fmaxf(red[0] * 5.9604644775390625e-08f, 1.17549435e-38f);
+}
+
+// pre-pass 2: u = round(x / grid) as a two's-complement integer with the sign bit flipped (a bias of 2^31),
+// which keeps the order of the values as unsigned integers: |u_q - u_k| is the distance in grid units.
+__global__ __launch_bounds__(256) void fixed_quantise(const float* __restrict__ q, const float* __restrict__ k,
+                                                        const float* __restrict__ gq, unsigned* __restrict__ uq,
+                                                        unsigned* __restrict__ uk, int64_t n, int H, int W, int64_t TH)
+{
+	for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+		const int64_t row = i / W;  // (b*T + t)*H + h
+		const float g = gq[(row / TH) * H + row % H];
+		uq[i] = (unsigned)(int)rintf(q[i] / g) ^ 0x80000000u;
+		uk[i] = (unsigned)(int)rintf(k[i] / g) ^ 0x80000000u;
+	}
+}
+
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
@@ -852,8 +927,9 @@ bool fwd_fast_ok(const float* q, const float* k, int64_t B, int64_t T, int64_t H
 
 // W: width of the rows the kernels read; W_scale: width the logits are scaled by (smaller when the rows are
 // zero-padded copies)
+// gq != nullptr: q and k are the fixed-point copies and gq their grids (widths 32 and 64 only)
 int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int64_t Tn, int64_t H, int64_t W,
-                    int64_t W_scale, hipStream_t st)
+                    int64_t W_scale, hipStream_t st, const float* gq = nullptr)
 {
 	// width 128 runs the pipelined width-64 kernel on half-heads (128 q registers per lane do not leave room
 	// for four waves per SIMD)
@@ -880,9 +956,20 @@ int launch_fwd_fast(const float* q, const float* k, float* attn, int64_t B, int6
 		break
 #define L1_FWD_PIPE_CASE(WV)                                                                                     \
 	case WV:                                                                                                     \
-		hipLaunchKernelGGL(dense_fwd_f32_pipe<WV>, grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, NH,      \
-		                   (int)s_chunk, scale, V);                                                              \
+		hipLaunchKernelGGL((dense_fwd_f32_pipe<WV, false>), grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, \
+		                   NH, (int)s_chunk, scale, V, (const float*)nullptr);                                   \
 		break
+	if (gq) {
+		if (V != 1 || (W != 32 && W != 64)) return L1ATTN_ERR_ARG;
+		if (W == 32)
+			hipLaunchKernelGGL((dense_fwd_f32_pipe<32, true>), grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, NH,
+			                   (int)s_chunk, scale, V, gq);
+		else
+			hipLaunchKernelGGL((dense_fwd_f32_pipe<64, true>), grid, block, 0, st, q, k, attn, (int)Tn, (int)H, n_hg, NH,
+			                   (int)s_chunk, scale, V, gq);
+		L1_LAUNCH_CHECK();
+		return L1ATTN_OK;
+	}
 	switch (W) {
 		L1_FWD_CASE(dense_fwd_f32_fast, 16); L1_FWD_PIPE_CASE(32);
 		L1_FWD_CASE(dense_fwd_f32_fast, 48); L1_FWD_PIPE_CASE(64);
@@ -1078,6 +1165,38 @@ int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn, int64_t
 		return launch_fwd_fast(qp, kp, attn, B, T, H, WP, W, st);
 	}
 	return launch_fwd_generic<float>(q, k, attn, B, T, H, W, st);
+}
+
+// Fixed-point forward (experimental, fp32 in and out): workspace = grids [B*H] (padded to 256 bytes), then the
+// fixed-point copies of q and k.
+static size_t fixed_grid_bytes(int64_t B, int64_t H) { return l1_align_up((size_t)(B * H) * sizeof(float), 256); }
+
+size_t l1attn_dense_fwd_fixed_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	if (!shape_ok(B, T, H, W) || B * T * H * W == 0) return 0;
+	return fixed_grid_bytes(B, H) + (size_t)2 * B * T * H * W * sizeof(float);
+}
+
+int l1attn_dense_fwd_fixed_f32(const float* q, const float* k, float* attn, int64_t B, int64_t T, int64_t H, int64_t W,
+                               void* workspace, size_t workspace_bytes, void* stream)
+{
+	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	if (B * T * T * H == 0) return L1ATTN_OK;
+	if (!q || !k || !attn) return L1ATTN_ERR_ARG;
+	if ((W != 32 && W != 64) || !fwd_fast_ok(q, k, B, T, H, W) || B * H > 2147483647LL) return L1ATTN_ERR_ARG;
+	if (!workspace || (((uintptr_t)workspace) & 15) || workspace_bytes < l1attn_dense_fwd_fixed_workspace_bytes(B, T, H, W))
+		return L1ATTN_ERR_WORKSPACE;
+	hipStream_t st = (hipStream_t)stream;
+	float* gq = (float*)workspace;
+	unsigned* uq = (unsigned*)((char*)workspace + fixed_grid_bytes(B, H));
+	const int64_t n = B * T * H * W;
+	unsigned* uk = uq + n;
+	hipLaunchKernelGGL(fixed_absmax, dim3((unsigned)(B * H)), dim3(256), 0, st, q, k, gq, (int)T, (int)H, (int)W);
+	L1_LAUNCH_CHECK();
+	const dim3 qgrid((unsigned)std::min<int64_t>(l1_cdiv(n, 256), 1 << 20));
+	hipLaunchKernelGGL(fixed_quantise, qgrid, dim3(256), 0, st, q, k, (const float*)gq, uq, uk, n, (int)H, (int)W, T * H);
+	L1_LAUNCH_CHECK();
+	return launch_fwd_fast((const float*)uq, (const float*)uk, attn, B, T, H, W, W, st, gq);
 }
 
 int l1attn_dense_fwd_f64(const double* q, const double* k, double* attn, int64_t B, int64_t T, int64_t H, int64_t W,

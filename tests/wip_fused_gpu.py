@@ -125,3 +125,33 @@ def test_probe_other_instructions_runs():
         assert L.l1attn_probe_valu_op(drv.ptr(out), 4, 3, op, drv.stream_of(out)) == 0
     torch.cuda.synchronize()
     assert L.l1attn_probe_valu_op(drv.ptr(out), 4, 3, 4, drv.stream_of(out)) == -1
+
+
+@pytest.mark.parametrize("shape,layernorm", [((2, 64, 4, 32), False), ((1, 100, 3, 64), False), ((2, 200, 16, 64), True),
+                                              ((1, 1100, 5, 32), False)])
+def test_fixed_point_forward_vs_oracle(shape, layernorm):
+    """Experimental fixed-point forward (one v_sad_u32 per pair-element) against the fp64 oracle, same
+    tolerance as the fp32 forward (1e-5 of the largest logit), beside the fp32 kernel's own error; exact
+    zeros on the diagonal when k == q; a head of zeros; bitwise repeatability."""
+    B, T, H, W = shape
+    print("case fixed-point forward", shape, layernorm, flush=True)
+    import _l1attn_hip as drv
+    q, k, _ = workloads.dense_inputs(B, T, H, W, seed=sum(shape), layernorm=layernorm)
+    q[:, :, 0, :] *= 37.0   # heads of different magnitude get different grids
+    ref = oracle.dense_fwd(q.double(), k.double())
+    a, = drv.dense_forward_fixed(q.cuda(), k.cuda())
+    a32, = drv.dense_forward(q.cuda(), k.cuda())
+    torch.cuda.synchronize()
+    e_fix, e_f32 = cf.rel_err(a.cpu(), ref), cf.rel_err(a32.cpu(), ref)
+    print("fixed", e_fix, "fp32", e_f32, flush=True)
+    assert e_fix <= F32_TOL
+    a2, = drv.dense_forward_fixed(q.cuda(), k.cuda())
+    assert torch.equal(a, a2)
+    d, = drv.dense_forward_fixed(q.cuda(), q.cuda())
+    assert torch.count_nonzero(torch.diagonal(d, dim1=1, dim2=2)) == 0
+    qz = q.clone()
+    qz[:, :, H - 1, :] = 0
+    z, = drv.dense_forward_fixed(qz.cuda(), qz.cuda())
+    assert torch.count_nonzero(z[..., H - 1]) == 0 and torch.isfinite(z).all()
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        drv.dense_forward_fixed(torch.zeros(1, 64, 2, 48).cuda(), torch.zeros(1, 64, 2, 48).cuda())
