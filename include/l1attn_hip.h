@@ -152,7 +152,7 @@ int l1attn_dense_fwd_fixed_f32(const float* q, const float* k, float* attn,
  * The reference has no single function for this; it is the composition its model code builds from
  * l1attn_cuda_drv.forward (a zero logit row appended, softmax over dim 1, 'bsdh,bshw->bdhw':
  * example-setfind/setfind.py:128-136, python/l1attn_sparse.py:488-506) and the form its README asks
- * for (README.md:21).  q,k [B,T,H,W]; v,vo [B,T,H,Wv].  Forward only.  Deterministic.
+ * for (README.md:21).  q,k [B,T,H,W]; v,vo [B,T,H,Wv].  Deterministic.  Backward: below.
  * f32: W == Wv in {16,32,64}, T >= 32 and 16-byte aligned pointers run the tiled kernel; every other
  * shape, and f64, a generic one (L1ATTN_ERR_RANGE when it would need 2^32 threads or more).
  */
@@ -160,6 +160,21 @@ int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* 
                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
 int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, double* vo, double* lse,
                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
+
+/*
+ * Backward of the fused forward, first stage.  With p[s,t] = exp(a[s,t] - lse[t]), dp[s,t] = v[s].dvo[t],
+ * S[t] = vo[t].dvo[t]:   dA[b,s,t,h] = p * (dp - S[t])  (gradient of the logits, dense layout [B,S,T,H])
+ * and dv[b,s,h,:] = sum_t p[s,t] * dvo[b,t,h,:].  dq and dk are then l1attn_dense_bwd_* of (dA, q, k).
+ * vo and lse are the forward's outputs.  dA is the only [B,T,T,H] tensor of the whole forward + backward
+ * (the unfused composition of example-setfind/setfind.py:128-136 keeps the logits, the weights and the
+ * gradients of both).  No counterpart in the reference.  Deterministic.  Shapes as l1attn_fused_fwd_*.
+ */
+int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k, const float* v,
+                               const float* vo, const float* lse, float* dA, float* dv,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
+int l1attn_fused_bwd_stage_f64(const double* dvo, const double* q, const double* k, const double* v,
+                               const double* vo, const double* lse, double* dA, double* dv,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
 
 /* -------------------------------------------------------------------------- edge lists */
 

@@ -64,6 +64,9 @@ def lib():
             f = getattr(L, "l1attn_fused_fwd_" + sfx)
             f.restype = _c_i
             f.argtypes = [_c_p] * 5 + [_c_i64] * 5 + [_c_p]
+            f = getattr(L, "l1attn_fused_bwd_stage_" + sfx)
+            f.restype = _c_i
+            f.argtypes = [_c_p] * 8 + [_c_i64] * 5 + [_c_p]
         L.l1attn_dense_column_ranks_f32.restype = _c_i
         L.l1attn_dense_column_ranks_f32.argtypes = [_c_p] * 4 + [_c_i64] * 4 + [_c_p]
         L.l1attn_expand_coo_workspace_bytes.restype = _c_sz
@@ -232,6 +235,33 @@ def dense_fused_forward(q, k, v, want_lse=False):
             ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse) if lse is not None else None, B, T, H, W, Wv, stream_of(q))
     check(rc, "l1attn_fused_fwd_" + sfx)
     return [vo, lse]
+
+
+def dense_fused_backward(dvo, q, k, v, vo, lse):
+    """Backward of dense_fused_forward -> [dq, dk, dv].  Stage one writes dA [B,T,T,H] (the gradient of the
+    logits, from dvo and the forward's vo and lse) and dv; dq and dk are the dense backward of dA."""
+    for x, n in ((dvo, "dvo"), (q, "q"), (k, "k"), (v, "v"), (vo, "vo"), (lse, "lse")):
+        check_input(x, n)
+    if q.dim() != 4 or q.shape != k.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
+        raise RuntimeError("q, k, v must be [batch, n_ctx, n_heads, width] tensors with equal leading dims")
+    _same_as(k, q, "k", "q")
+    _same_as(dvo, v, "dvo", "v")
+    _same_as(vo, v, "vo", "v")
+    B, T, H, W = q.shape
+    if v.dtype != q.dtype or v.device != q.device or tuple(lse.shape) != (B, T, H) or lse.dtype != q.dtype \
+            or lse.device != q.device:
+        raise RuntimeError("v must have the dtype and device of q, and lse must be the [batch, n_ctx, n_heads] "
+                           "tensor the forward returned")
+    sfx = sfx_of(q)
+    dA = torch.empty((B, T, T, H), dtype=q.dtype, device=q.device)
+    dv = torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        rc = getattr(lib(), "l1attn_fused_bwd_stage_" + sfx)(
+            ptr(dvo), ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse), ptr(dA), ptr(dv), B, T, H, W, v.shape[3],
+            stream_of(q))
+    check(rc, "l1attn_fused_bwd_stage_" + sfx)
+    dq, dk = dense_backward(dA, q, k)
+    return [dq, dk, dv]
 
 
 # ------------------------------------------------------------------------------- edge lists

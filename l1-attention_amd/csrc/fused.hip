@@ -111,6 +111,163 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restric
 	}
 }
 
+// ------------------------------------------------------------------------------------------ backward
+// With p[s,t] = exp(a[s,t] - lse[t]), dp[s,t] = v[s].dvo[t] and S[t] = vo[t].dvo[t] (= sum_s p*dp):
+//   dA[s,t] = p * (dp - S[t])                  gradient of the logits, written in the dense layout [B,S,T,H]
+//   dv[s,:] = sum_t p[s,t] * dvo[t,:]
+// dq and dk then come from the dense backward on dA.  Only dA is ever held of the four [B,T,T,H] tensors
+// (logits, weights and their two gradients) that the unfused composition keeps.
+
+// any shape: one thread per dA element
+template <typename T>
+__global__ __launch_bounds__(256) void fused_bwd_da_generic(const T* __restrict__ dvo, const T* __restrict__ q,
+                                                              const T* __restrict__ k, const T* __restrict__ v,
+                                                              const T* __restrict__ vo, const T* __restrict__ lse,
+                                                              T* __restrict__ dA, int64_t B, int64_t Tn, int64_t H,
+                                                              int64_t W, int64_t Wv, T scale)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= B * Tn * Tn * H) return;
+	const int64_t h = idx % H, t = (idx / H) % Tn, s = (idx / (H * Tn)) % Tn, b = idx / (H * Tn * Tn);
+	const T* qp = q + ((b * Tn + t) * H + h) * W;
+	const T* kp = k + ((b * Tn + s) * H + h) * W;
+	T f = 0;
+	for (int64_t w = 0; w < W; w++) f += fabs_t(qp[w] - kp[w]);
+	const T* vp = v + ((b * Tn + s) * H + h) * Wv;
+	const T* op = vo + ((b * Tn + t) * H + h) * Wv;
+	const T* gp = dvo + ((b * Tn + t) * H + h) * Wv;
+	T dp = 0, S = 0;
+	for (int64_t w = 0; w < Wv; w++) { dp += vp[w] * gp[w]; S += op[w] * gp[w]; }
+	dA[idx] = exp_t(f * scale - lse[(b * Tn + t) * H + h]) * (dp - S);
+}
+
+// any shape: one thread per dv element, dst tokens summed in ascending order
+template <typename T>
+__global__ __launch_bounds__(256) void fused_bwd_dv_generic(const T* __restrict__ dvo, const T* __restrict__ q,
+                                                              const T* __restrict__ k, const T* __restrict__ lse,
+                                                              T* __restrict__ dv, int64_t B, int64_t Tn, int64_t H,
+                                                              int64_t W, int64_t Wv, T scale)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= B * Tn * H * Wv) return;
+	const int64_t wv = idx % Wv, h = (idx / Wv) % H, s = (idx / (Wv * H)) % Tn, b = idx / (Wv * H * Tn);
+	const T* kp = k + ((b * Tn + s) * H + h) * W;
+	T acc = 0;
+	for (int64_t t = 0; t < Tn; t++) {
+		const T* qp = q + ((b * Tn + t) * H + h) * W;
+		T f = 0;
+		for (int64_t w = 0; w < W; w++) f += fabs_t(qp[w] - kp[w]);
+		acc += exp_t(f * scale - lse[(b * Tn + t) * H + h]) * dvo[((b * Tn + t) * H + h) * Wv + wv];
+	}
+	dv[idx] = acc;
+}
+
+// Tiled dA: the forward's mapping (wave = head, lane = dst token t).  A lane keeps q[t], dvo[t] and S[t]; the
+// k and v rows of the src token are wave-uniform.  Per pair-element v_sub, v_add |x|, v_fmac.
+// The stores are 4 bytes per lane at a pitch of H floats (one head of the [t][h] plane per wave).
+template <int W>
+__global__ __launch_bounds__(256) void fused_bwd_da_tile(const float* __restrict__ dvo, const float* __restrict__ q,
+                                                           const float* __restrict__ k, const float* __restrict__ v,
+                                                           const float* __restrict__ vo, const float* __restrict__ lse,
+                                                           float* __restrict__ dA, int Tn, int H, int n_hg, int NH,
+                                                           float scale)
+{
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.y / n_hg, hg = lb.y % n_hg;
+	const int h_raw = hg * NH + wave;
+	const int h = min(h_raw, H - 1);
+	const int t_raw = lb.x * 64 + lane;
+	const int t = min(t_raw, Tn - 1);
+	const bool store = h_raw < H && t_raw < Tn;
+
+	float qr[W], gr[W];
+	float S = 0.0f;
+	{
+		const int64_t off = (((int64_t)b * Tn + t) * H + h) * (int64_t)W;
+		const float4* qp = reinterpret_cast<const float4*>(q + off);
+		const float4* gp = reinterpret_cast<const float4*>(dvo + off);
+		const float4* op = reinterpret_cast<const float4*>(vo + off);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = qp[w4], g = gp[w4], o = op[w4];
+			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
+			gr[w4 * 4 + 0] = g.x; gr[w4 * 4 + 1] = g.y; gr[w4 * 4 + 2] = g.z; gr[w4 * 4 + 3] = g.w;
+			S += o.x * g.x; S += o.y * g.y; S += o.z * g.z; S += o.w * g.w;
+		}
+	}
+	const float l = lse[((int64_t)b * Tn + t) * H + h];
+	const int64_t row = (int64_t)H * W;
+	const float* kp = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	const float* vp = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	float* out = dA + (((int64_t)b * Tn) * Tn + t) * H + h;  // src token 0
+	const int64_t pitch = (int64_t)Tn * H;
+	for (int s = 0; s < Tn; s++) {
+		float a = 0.0f, dp = 0.0f;
+#pragma unroll
+		for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
+#pragma unroll
+		for (int w = 0; w < W; w++) dp += gr[w] * vp[w];
+		if (store) *out = expf(a * scale - l) * (dp - S);
+		out += pitch;
+		kp += row;
+		vp += row;
+	}
+}
+
+// Tiled dv: wave = head, lane = src token s.  A lane keeps k[s] and its dv row; the q and dvo rows and lse of the
+// dst token are wave-uniform.  Per pair-element v_sub, v_add |x|, v_fmac; dst tokens in ascending order.
+template <int W>
+__global__ __launch_bounds__(256) void fused_bwd_dv_tile(const float* __restrict__ dvo, const float* __restrict__ q,
+                                                           const float* __restrict__ k, const float* __restrict__ lse,
+                                                           float* __restrict__ dv, int Tn, int H, int n_hg, int NH,
+                                                           float scale)
+{
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.y / n_hg, hg = lb.y % n_hg;
+	const int h_raw = hg * NH + wave;
+	const int h = min(h_raw, H - 1);
+	const int s_raw = lb.x * 64 + lane;
+	const int s = min(s_raw, Tn - 1);
+	const bool store = h_raw < H && s_raw < Tn;
+
+	float kr[W], acc[W];
+	{
+		const float4* kp = reinterpret_cast<const float4*>(k + (((int64_t)b * Tn + s) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = kp[w4];
+			kr[w4 * 4 + 0] = x.x; kr[w4 * 4 + 1] = x.y; kr[w4 * 4 + 2] = x.z; kr[w4 * 4 + 3] = x.w;
+		}
+#pragma unroll
+		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+	}
+	const int64_t row = (int64_t)H * W;
+	const float* qp = q + (((int64_t)b * Tn) * H + h) * (int64_t)W;    // dst token 0 of this (b,h): wave-uniform
+	const float* gp = dvo + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	const float* lp = lse + ((int64_t)b * Tn) * H + h;
+	for (int t = 0; t < Tn; t++) {
+		float a = 0.0f;
+#pragma unroll
+		for (int w = 0; w < W; w++) a += fabsf(qp[w] - kr[w]);
+		const float p = expf(a * scale - *lp);
+#pragma unroll
+		for (int w = 0; w < W; w++) acc[w] += p * gp[w];
+		qp += row;
+		gp += row;
+		lp += H;
+	}
+	if (store) {
+		float4* op = reinterpret_cast<float4*>(dv + (((int64_t)b * Tn + s) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++)
+			op[w4] = make_float4(acc[w4 * 4 + 0], acc[w4 * 4 + 1], acc[w4 * 4 + 2], acc[w4 * 4 + 3]);
+	}
+}
+
 bool shape_ok(int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv)
 {
 	return B >= 0 && T >= 0 && H >= 0 && W >= 1 && Wv >= 1;
@@ -125,6 +282,22 @@ int launch_generic(const T* q, const T* k, const T* v, T* vo, T* lse, int64_t B,
 	const T scale = (T)(-1.0 / sqrt((double)W));
 	hipLaunchKernelGGL(fused_fwd_generic<T>, dim3((unsigned)l1_cdiv(n, 256)), dim3(256), 0, st, q, k, v, vo, lse, B, Tn,
 	                   H, W, Wv, scale);
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+template <typename T>
+int launch_bwd_generic(const T* dvo, const T* q, const T* k, const T* v, const T* vo, const T* lse, T* dA, T* dv,
+                       int64_t B, int64_t Tn, int64_t H, int64_t W, int64_t Wv, hipStream_t st)
+{
+	const int64_t na = B * Tn * Tn * H, nv = B * Tn * H * Wv;
+	if (na >= ((int64_t)1 << 32) || nv >= ((int64_t)1 << 32)) return L1ATTN_ERR_RANGE;  // one thread per element
+	const T scale = (T)(-1.0 / sqrt((double)W));
+	hipLaunchKernelGGL(fused_bwd_da_generic<T>, dim3((unsigned)l1_cdiv(na, 256)), dim3(256), 0, st, dvo, q, k, v, vo,
+	                   lse, dA, B, Tn, H, W, Wv, scale);
+	L1_LAUNCH_CHECK();
+	hipLaunchKernelGGL(fused_bwd_dv_generic<T>, dim3((unsigned)l1_cdiv(nv, 256)), dim3(256), 0, st, dvo, q, k, lse, dv,
+	                   B, Tn, H, W, Wv, scale);
 	L1_LAUNCH_CHECK();
 	return L1ATTN_OK;
 }
@@ -171,6 +344,53 @@ int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, doub
 	if (B * T * H == 0) return L1ATTN_OK;
 	if (!q || !k || !v || !vo) return L1ATTN_ERR_ARG;
 	return launch_generic<double>(q, k, v, vo, lse, B, T, H, W, Wv, (hipStream_t)stream);
+}
+
+// First stage of the fused backward: dA [B,S,T,H] (gradient of the logits) and dv from dvo and the forward's
+// vo and lse.  dq and dk follow from l1attn_dense_bwd_* on dA, q, k.
+int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k, const float* v, const float* vo,
+                               const float* lse, float* dA, float* dv, int64_t B, int64_t T, int64_t H, int64_t W,
+                               int64_t Wv, void* stream)
+{
+	if (!shape_ok(B, T, H, W, Wv)) return L1ATTN_ERR_ARG;
+	if (B * T * H == 0) return L1ATTN_OK;
+	if (!dvo || !q || !k || !v || !vo || !lse || !dA || !dv) return L1ATTN_ERR_ARG;
+	hipStream_t st = (hipStream_t)stream;
+	const bool aligned = ((((uintptr_t)dvo) | ((uintptr_t)q) | ((uintptr_t)k) | ((uintptr_t)v) | ((uintptr_t)vo) |
+	                       ((uintptr_t)dv)) & 15) == 0;
+	const int NH = (int)(H < 4 ? H : 4);
+	const int64_t n_hg = l1_cdiv(H, NH);
+	const bool tiled = aligned && W == Wv && (W == 16 || W == 32 || W == 64) && T >= 32 && T <= (1 << 30) &&
+	                   B * n_hg <= 65535 && H <= 65535;
+	if (!tiled) return launch_bwd_generic<float>(dvo, q, k, v, vo, lse, dA, dv, B, T, H, W, Wv, st);
+	const float scale = (float)(-1.0 / sqrt((double)W));
+	const dim3 grid((unsigned)l1_cdiv(T, 64), (unsigned)(B * n_hg), 1), block(64 * NH);
+#define L1_FUSED_BWD_CASE(WV)                                                                                       \
+	case WV:                                                                                                        \
+		hipLaunchKernelGGL(fused_bwd_da_tile<WV>, grid, block, 0, st, dvo, q, k, v, vo, lse, dA, (int)T, (int)H,     \
+		                   (int)n_hg, NH, scale);                                                                   \
+		hipLaunchKernelGGL(fused_bwd_dv_tile<WV>, grid, block, 0, st, dvo, q, k, lse, dv, (int)T, (int)H, (int)n_hg,  \
+		                   NH, scale);                                                                              \
+		break
+	switch (W) {
+		L1_FUSED_BWD_CASE(16);
+		L1_FUSED_BWD_CASE(32);
+		L1_FUSED_BWD_CASE(64);
+	default: return L1ATTN_ERR_ARG;
+	}
+#undef L1_FUSED_BWD_CASE
+	L1_LAUNCH_CHECK();
+	return L1ATTN_OK;
+}
+
+int l1attn_fused_bwd_stage_f64(const double* dvo, const double* q, const double* k, const double* v, const double* vo,
+                               const double* lse, double* dA, double* dv, int64_t B, int64_t T, int64_t H, int64_t W,
+                               int64_t Wv, void* stream)
+{
+	if (!shape_ok(B, T, H, W, Wv)) return L1ATTN_ERR_ARG;
+	if (B * T * H == 0) return L1ATTN_OK;
+	if (!dvo || !q || !k || !v || !vo || !lse || !dA || !dv) return L1ATTN_ERR_ARG;
+	return launch_bwd_generic<double>(dvo, q, k, v, vo, lse, dA, dv, B, T, H, W, Wv, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -42,18 +42,23 @@ class L1Attn(nn.Module):
 
 
 class L1AttnFusedFn(Function):
-    """L1 attention with the value sum fused in (forward only): softmax over the src tokens of the L1
-    logits with the no-op zero logit, times v, without the [B,T,T,H] tensor.  Equals
+    """L1 attention with the value sum fused in: softmax over the src tokens of the L1 logits with the no-op
+    zero logit, times v, without the [B,T,T,H] logits.  Equals
     einsum('bsdh,bshw->bdhw', softmax(cat(L1Attn()(q,k), zeros), 1)[:, :-1], v), the composition of
-    example-setfind/setfind.py:128-136.  The reference has no such function (README.md:21 asks for it)."""
+    example-setfind/setfind.py:128-136.  The reference has no such function (README.md:21 asks for it).
+    The backward holds one [B,T,T,H] tensor (the gradient of the logits) where the composition holds four."""
     @staticmethod
     def forward(ctx, q, k, v):
-        vo, _ = _drv.dense_fused_forward(q.contiguous(), k.contiguous(), v.contiguous())
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        vo, lse = _drv.dense_fused_forward(q, k, v, want_lse=True)
+        ctx.save_for_backward(q, k, v, vo, lse)
         return vo
 
     @staticmethod
     def backward(ctx, d_vo):
-        raise RuntimeError("L1AttnFused has no backward: use L1Attn with softmax and einsum for training")
+        q, k, v, vo, lse = ctx.saved_tensors[:5]
+        d_q, d_k, d_v = _drv.dense_fused_backward(d_vo.contiguous(), q, k, v, vo, lse)
+        return d_q, d_k, d_v
 
 
 class L1AttnFused(nn.Module):

@@ -1,8 +1,9 @@
 // TEST INFRASTRUCTURE: runs l1attn_fused_fwd_f32 / _f64 of csrc/fused.hip, compiled for the host with
 // the stand-in header next to this file, on inputs read from a file, and writes vo and lse.
 //   run_fused <in> <out> <f32|f64> <misalign>
-// in : int64 B,T,H,W,Wv then q,k [B,T,H,W] and v [B,T,H,Wv] in the chosen type
-// out: vo [B,T,H,Wv], lse [B,T,H], then one int64: threads run
+// in : int64 B,T,H,W,Wv then q,k [B,T,H,W], v [B,T,H,Wv] and dvo [B,T,H,Wv] in the chosen type
+// out: vo [B,T,H,Wv], lse [B,T,H], one int64 (threads the forward ran), then the backward's first stage on
+//      the forward's own vo and lse: dA [B,T,T,H], dv [B,T,H,Wv], one int64 (threads it ran)
 // Buffers are malloc'ed at their exact sizes, so AddressSanitizer reports any access outside them.
 // misalign = 1 offsets every buffer by one element (the library then has to take its generic kernel).
 #include "../../l1-attention_amd/csrc/fused.hip"
@@ -27,9 +28,25 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, bool f32, int mis)
 	if (rc) return 10 + (rc < 0 ? -rc : rc);
 	fwrite(vo, sizeof(T), nv, fo);
 	fwrite(lse, sizeof(T), nl, fo);
-	const int64_t n = emu::n_threads_run;
+	int64_t n = emu::n_threads_run;
+	fwrite(&n, sizeof(n), 1, fo);
+	const size_t na = (size_t)(B * Tn * Tn * H);
+	T *dvo = alloc(nv), *dA = alloc(na), *dv = alloc(nv);
+	if (fread(dvo, sizeof(T), nv, fi) != nv) return 3;
+	emu::n_threads_run = 0;
+	if (f32) rc = l1attn_fused_bwd_stage_f32((const float*)dvo, (const float*)q, (const float*)k, (const float*)v,
+	                                         (const float*)vo, (const float*)lse, (float*)dA, (float*)dv, B, Tn, H, W,
+	                                         Wv, nullptr);
+	else rc = l1attn_fused_bwd_stage_f64((const double*)dvo, (const double*)q, (const double*)k, (const double*)v,
+	                                     (const double*)vo, (const double*)lse, (double*)dA, (double*)dv, B, Tn, H, W,
+	                                     Wv, nullptr);
+	if (rc) return 20 + (rc < 0 ? -rc : rc);
+	fwrite(dA, sizeof(T), na, fo);
+	fwrite(dv, sizeof(T), nv, fo);
+	n = emu::n_threads_run;
 	fwrite(&n, sizeof(n), 1, fo);
 	free(q - mis); free(k - mis); free(v - mis); free(vo - mis); free(lse - mis);
+	free(dvo - mis); free(dA - mis); free(dv - mis);
 	return 0;
 }
 

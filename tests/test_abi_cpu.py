@@ -310,6 +310,12 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
         drv.dense_fused_forward(q, k, torch.zeros(B, T + 1, H, Wv))
     with pytest.raises(RuntimeError, match="share dtype"):
         drv.dense_fused_forward(q, k, v.double())
+    grads = drv.dense_fused_backward(torch.zeros_like(v), q, k, v, vo, lse)
+    assert [g.shape for g in grads] == [q.shape, k.shape, v.shape]
+    with pytest.raises(RuntimeError, match="lse must be"):
+        drv.dense_fused_backward(torch.zeros_like(v), q, k, v, vo, lse[:, :-1])
+    with pytest.raises(RuntimeError, match="dvo must have"):
+        drv.dense_fused_backward(torch.zeros(B, T, H, Wv + 1), q, k, v, vo, lse)
     plan = drv.plan_for(coo, T)
     assert (plan.E, plan.T, plan.max_dst_deg, plan.max_src_deg) == (E, T, 3, 2)
     assert drv.plan_for(coo, T) is plan                      # cached on the tensor
@@ -382,9 +388,12 @@ def test_operator_modules_autograd_plumbing_without_a_gpu(monkeypatch):
     vo = l1attn_sparse_bidi_cuda.L1AttnSparseBidi()(vf, vb, q, k, coo, 2, True)
     vo.sum().backward()
     assert all(t.grad is not None and t.grad.shape == t.shape for t in (vf, vb, q, k))
-    # the fused forward has no backward and says so
+    # the fused operator: forward saves vo and lse, backward returns three gradients
     q, k, v = mk(B, T, H, W), mk(B, T, H, W), mk(B, T, H, W)
+    del _FakeLib.calls[:]
     vo = l1attn_cuda.L1AttnFused()(q, k, v)
     assert vo.shape == v.shape
-    with pytest.raises(RuntimeError, match="no backward"):
-        vo.sum().backward()
+    vo.sum().backward()
+    assert all(t.grad is not None and t.grad.shape == t.shape for t in (q, k, v))
+    assert [c for c in _FakeLib.calls if not c.endswith("_bytes")] == \
+        ["l1attn_fused_fwd_f32", "l1attn_fused_bwd_stage_f32", "l1attn_dense_bwd_f32"]

@@ -1,4 +1,4 @@
-"""CPU run of the fused forward's kernels (csrc/fused.hip compiled with g++ against the host-only
+"""CPU run of the fused operator's kernels (forward and the backward's first stage) (csrc/fused.hip compiled with g++ against the host-only
 stand-in header tests/cpu_emu/hip/hip_runtime.h, every GPU thread executed in turn) under
 AddressSanitizer and UBSan, checked against the oracle.
 
@@ -33,24 +33,35 @@ def runner(tmp_path_factory):
 
 
 def _run(exe, tmp_path, q, k, v, misalign=0):
+    """-> dict: vo, lse, threads (forward), dA, dv, bwd_threads (first stage of the backward on a seeded dvo),
+    and dvo itself."""
     B, T, H, W = q.shape
     Wv = v.shape[3]
     kind = "f32" if q.dtype == torch.float32 else "f64"
+    dvo = torch.randn(B, T, H, Wv, generator=torch.Generator().manual_seed(99), dtype=q.dtype)
     fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
     with open(fin, "wb") as f:
         f.write(struct.pack("5q", B, T, H, W, Wv))
-        for x in (q, k, v):
+        for x in (q, k, v, dvo):
             f.write(x.contiguous().numpy().tobytes())
     env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
     r = subprocess.run([exe, fin, fout, kind, str(misalign)], env=env, capture_output=True, text=True)
     assert r.returncode == 0, (r.returncode, r.stderr[-2000:])
     raw = open(fout, "rb").read()
     dt = np.float32 if kind == "f32" else np.float64
-    nv, nl = B * T * H * Wv, B * T * H
-    vo = torch.from_numpy(np.frombuffer(raw, dt, nv).copy()).view(B, T, H, Wv)
-    lse = torch.from_numpy(np.frombuffer(raw, dt, nl, nv * dt().itemsize).copy()).view(B, T, H)
-    threads = struct.unpack("q", raw[-8:])[0]
-    return vo, lse, threads
+    isz = dt().itemsize
+    out, pos = {"dvo": dvo}, 0
+    for name, shape in (("vo", (B, T, H, Wv)), ("lse", (B, T, H)), ("threads", None), ("dA", (B, T, T, H)),
+                        ("dv", (B, T, H, Wv)), ("bwd_threads", None)):
+        if shape is None:
+            out[name] = struct.unpack_from("q", raw, pos)[0]
+            pos += 8
+        else:
+            n = int(np.prod(shape))
+            out[name] = torch.from_numpy(np.frombuffer(raw, dt, n, pos).copy()).view(*shape)
+            pos += n * isz
+    assert pos == len(raw)
+    return out
 
 
 def _ref(q, k, v):
@@ -58,6 +69,22 @@ def _ref(q, k, v):
     if q.shape[3] == v.shape[3]:
         return oracle.fused_fwd(q, k, v)
     return cf.dense_then_value(q, k, v, noop=True), (1.0 + cf.dense_attn(q, k).exp().sum(1)).log()
+
+
+def _check_backward(r, q, k, v, tol):
+    """dA against torch autograd through the closed form (gradient of vo.dvo with respect to the logits), dv
+    against autograd, and dq, dk = the oracle's dense backward of the emulated dA against autograd."""
+    q, k, v, dvo = (x.double() for x in (q, k, v, r["dvo"]))
+    a = cf.dense_attn(q, k).requires_grad_()
+    vd = v.clone().requires_grad_()
+    e = a.exp()
+    vo = torch.einsum("bsdh,bshw->bdhw", e / (1.0 + e.sum(1, keepdim=True)), vd)
+    dA_ref, dv_ref = torch.autograd.grad(vo, (a, vd), dvo)
+    assert cf.rel_err(r["dA"], dA_ref) <= tol and cf.rel_err(r["dv"], dv_ref) <= tol
+    qd, kd = q.clone().requires_grad_(), k.clone().requires_grad_()
+    dq_ref, dk_ref = torch.autograd.grad(cf.dense_then_value(qd, kd, v, noop=True), (qd, kd), dvo)
+    dq, dk = oracle.dense_bwd(r["dA"].double(), q, k)
+    assert cf.rel_err(dq, dq_ref) <= tol and cf.rel_err(dk, dk_ref) <= tol
 
 
 TILED = [
@@ -70,15 +97,17 @@ TILED = [
 
 
 @pytest.mark.parametrize("shape", TILED)
-def test_fused_tiled_kernel_on_cpu(runner, tmp_path, shape):
+def test_fused_tiled_kernels_on_cpu(runner, tmp_path, shape):
     B, T, H, W = shape
     g = torch.Generator().manual_seed(sum(shape))
     q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
-    vo, lse, threads = _run(runner, tmp_path, q, k, v)
+    r = _run(runner, tmp_path, q, k, v)
     NH = min(H, 4)
-    assert threads == -(-T // 64) * B * -(-H // NH) * 64 * NH  # the tiled kernel's launch, not the generic one's
+    launch = -(-T // 64) * B * -(-H // NH) * 64 * NH  # a tiled kernel's launch, not a generic one's
+    assert r["threads"] == launch and r["bwd_threads"] == 2 * launch
     ref, ref_lse = _ref(q, k, v)
-    assert cf.rel_err(vo, ref) <= 1e-5 and cf.rel_err(lse, ref_lse) <= 1e-5
+    assert cf.rel_err(r["vo"], ref) <= 1e-5 and cf.rel_err(r["lse"], ref_lse) <= 1e-5
+    _check_backward(r, q, k, v, 1e-4)
 
 
 GENERIC = [
@@ -88,24 +117,28 @@ GENERIC = [
 
 
 @pytest.mark.parametrize("shape", GENERIC)
-def test_fused_generic_kernel_on_cpu(runner, tmp_path, shape):
+def test_fused_generic_kernels_on_cpu(runner, tmp_path, shape):
     B, T, H, W, Wv = shape
     g = torch.Generator().manual_seed(sum(shape))
     q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))
     v = torch.randn(B, T, H, Wv, generator=g)
     ref, ref_lse = _ref(q, k, v)
-    vo, lse, threads = _run(runner, tmp_path, q, k, v)
-    assert threads == -(-(B * T * H * Wv) // 256) * 256
-    assert cf.rel_err(vo, ref) <= 1e-5 and cf.rel_err(lse, ref_lse) <= 1e-5
-    vo, lse, _ = _run(runner, tmp_path, q.double(), k.double(), v.double())
-    assert cf.rel_err(vo, ref) <= 1e-12 and cf.rel_err(lse, ref_lse) <= 1e-12
+    r = _run(runner, tmp_path, q, k, v)
+    up = lambda n: -(-n // 256) * 256
+    assert r["threads"] == up(B * T * H * Wv) and r["bwd_threads"] == up(B * T * T * H) + up(B * T * H * Wv)
+    assert cf.rel_err(r["vo"], ref) <= 1e-5 and cf.rel_err(r["lse"], ref_lse) <= 1e-5
+    _check_backward(r, q, k, v, 1e-4)
+    r = _run(runner, tmp_path, q.double(), k.double(), v.double())
+    assert cf.rel_err(r["vo"], ref) <= 1e-12 and cf.rel_err(r["lse"], ref_lse) <= 1e-12
+    _check_backward(r, q, k, v, 1e-11)
 
 
-def test_fused_unaligned_buffers_take_the_generic_kernel(runner, tmp_path):
+def test_fused_unaligned_buffers_take_the_generic_kernels(runner, tmp_path):
     B, T, H, W = 1, 64, 2, 32
     g = torch.Generator().manual_seed(5)
     q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
-    vo, lse, threads = _run(runner, tmp_path, q, k, v, misalign=1)
-    assert threads == B * T * H * W  # one thread per output element
+    r = _run(runner, tmp_path, q, k, v, misalign=1)
+    assert r["threads"] == B * T * H * W  # one thread per output element
     ref, ref_lse = _ref(q, k, v)
-    assert cf.rel_err(vo, ref) <= 1e-5 and cf.rel_err(lse, ref_lse) <= 1e-5
+    assert cf.rel_err(r["vo"], ref) <= 1e-5 and cf.rel_err(r["lse"], ref_lse) <= 1e-5
+    _check_backward(r, q, k, v, 1e-4)
