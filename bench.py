@@ -194,8 +194,36 @@ def extra_legs():
         ms_c = time_gpu(composed, 2 if big else 5, warm=1)
         err = float((fused(q, k, v) - composed()).abs().max() / composed().abs().max())
         N = B * T * T * H * W
+        # forward + backward, and the peak memory each route adds to the inputs
+        x = [t.clone().requires_grad_() for t in (q, k, v)]
+        dvo = torch.randn_like(v)
+
+        def train(fn):
+            for t in x:
+                t.grad = None
+            fn().backward(dvo)
+
+        def fused_step():
+            train(lambda: fused(*x))
+
+        def composed_step():
+            def f():
+                a = plain(x[0], x[1])
+                a = torch.cat((a, torch.zeros(B, 1, T, H, device=dev)), 1)
+                return torch.einsum("bsdh,bshw->bdhw", torch.softmax(a, 1)[:, :T], x[2])
+            train(f)
+
+        steps = {}
+        for label, fn in (("fused", fused_step), ("composed", composed_step)):
+            torch.cuda.empty_cache()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()
+            ms = time_gpu(fn, 2 if big else 5, warm=1)
+            steps[label] = {"fwd_bwd_ms": ms, "peak_extra_GiB": (torch.cuda.max_memory_allocated() - base) / 2.0 ** 30}
+        del x, dvo
         res["fused_forward"][name] = {
             "fused_ms": ms_f, "composed_ms": ms_c, "speedup": ms_c / ms_f, "max_rel_diff": err,
+            "fwd_bwd": steps,
             "fused_tops": 3 * N / ms_f / 1e9, "frac_of_valu_peak": 3 * N / ms_f / 1e9 / P_VALU_TOPS,
             "note": "3 algorithmic ops per pair-element (sub, abs-accumulate, multiply-accumulate)"}
         log(name, json.dumps(res["fused_forward"][name]))
