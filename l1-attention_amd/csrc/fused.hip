@@ -162,25 +162,33 @@ __global__ __launch_bounds__(256) void fused_bwd_dv_generic(const T* __restrict_
 	dv[idx] = acc;
 }
 
-// Tiled dA: the forward's mapping (wave = head, lane = dst token t).  A lane keeps q[t], dvo[t] and S[t]; the
-// k and v rows of the src token are wave-uniform.  Per pair-element v_sub, v_add |x|, v_fmac.
-// The stores are 4 bytes per lane at a pitch of H floats (one head of the [t][h] plane per wave).
+// Tiled dA: the forward's mapping (wave = head, lane = dst token t), up to eight heads per workgroup.  A lane
+// keeps q[t], dvo[t] and S[t]; the k and v rows of the src token are wave-uniform.  Per pair-element v_sub,
+// v_add |x|, v_fmac.  The values of DA_SJ src rows are transposed through LDS so that the workgroup stores
+// runs of NH consecutive heads per (s,t) (32 bytes with eight heads) instead of 4 bytes per lane at a pitch of
+// H floats.  blockDim.x = 64*NH: one element of the [64 t x NH] plane per thread and src row.
+constexpr int DA_SJ = 8;    // src rows between two flushes
+constexpr int DA_NH = 8;    // most heads per workgroup
+
 template <int W>
-__global__ __launch_bounds__(256) void fused_bwd_da_tile(const float* __restrict__ dvo, const float* __restrict__ q,
-                                                           const float* __restrict__ k, const float* __restrict__ v,
-                                                           const float* __restrict__ vo, const float* __restrict__ lse,
-                                                           float* __restrict__ dA, int Tn, int H, int n_hg, int NH,
-                                                           float scale)
+__global__ __launch_bounds__(64 * DA_NH) void fused_bwd_da_tile(const float* __restrict__ dvo,
+                                                                  const float* __restrict__ q,
+                                                                  const float* __restrict__ k,
+                                                                  const float* __restrict__ v,
+                                                                  const float* __restrict__ vo,
+                                                                  const float* __restrict__ lse,
+                                                                  float* __restrict__ dA, int Tn, int H, int n_hg,
+                                                                  int NH, float scale)
 {
+	__shared__ float tile[DA_SJ][64 * (DA_NH + 1)];  // [src row][t * (NH+1) + head]: the odd pitch spreads the banks
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const LogicalBlock lb = xcd_remap();
 	const int b = lb.y / n_hg, hg = lb.y % n_hg;
-	const int h_raw = hg * NH + wave;
-	const int h = min(h_raw, H - 1);
-	const int t_raw = lb.x * 64 + lane;
-	const int t = min(t_raw, Tn - 1);
-	const bool store = h_raw < H && t_raw < Tn;
+	const int h = min(hg * NH + wave, H - 1);  // surplus waves of the last group redo head H-1, never stored
+	const int t0 = lb.x * 64;
+	const int t = min(t0 + lane, Tn - 1);      // surplus lanes of the last tile redo token Tn-1, never stored
+	const int PH = NH + 1;
 
 	float qr[W], gr[W];
 	float S = 0.0f;
@@ -199,20 +207,31 @@ __global__ __launch_bounds__(256) void fused_bwd_da_tile(const float* __restrict
 	}
 	const float l = lse[((int64_t)b * Tn + t) * H + h];
 	const int64_t row = (int64_t)H * W;
-	const float* kp = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;
-	const float* vp = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
-	float* out = dA + (((int64_t)b * Tn) * Tn + t) * H + h;  // src token 0
+	const float* kb = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;  // src token 0 of this (b,h): wave-uniform
+	const float* vb = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	// role of this thread in the flush: element (o_t, o_h) of the [64 t x NH] plane
+	const int o_t = threadIdx.x / NH, o_h = threadIdx.x % NH;
+	const bool o_ok = (t0 + o_t < Tn) && (hg * NH + o_h < H);
+	float* const o_base = dA + (((int64_t)b * Tn) * Tn + (t0 + o_t)) * H + hg * NH + o_h;  // src token 0
 	const int64_t pitch = (int64_t)Tn * H;
-	for (int s = 0; s < Tn; s++) {
-		float a = 0.0f, dp = 0.0f;
+	for (int s0 = 0; s0 < Tn; s0 += DA_SJ) {
+#pragma unroll 1
+		for (int j = 0; j < DA_SJ; j++) {
+			const int s = min(s0 + j, Tn - 1);  // rows past the end are computed on the last row and not stored
+			const float* kp = kb + s * row;
+			const float* vp = vb + s * row;
+			float a = 0.0f, dp = 0.0f;
 #pragma unroll
-		for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
+			for (int w = 0; w < W; w++) a += fabsf(qr[w] - kp[w]);
 #pragma unroll
-		for (int w = 0; w < W; w++) dp += gr[w] * vp[w];
-		if (store) *out = expf(a * scale - l) * (dp - S);
-		out += pitch;
-		kp += row;
-		vp += row;
+			for (int w = 0; w < W; w++) dp += gr[w] * vp[w];
+			tile[j][lane * PH + wave] = expf(a * scale - l) * (dp - S);
+		}
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < DA_SJ; j++)
+			if (o_ok && s0 + j < Tn) o_base[(int64_t)(s0 + j) * pitch] = tile[j][o_t * PH + o_h];
+		__syncthreads();
 	}
 }
 
@@ -365,10 +384,14 @@ int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k,
 	if (!tiled) return launch_bwd_generic<float>(dvo, q, k, v, vo, lse, dA, dv, B, T, H, W, Wv, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
 	const dim3 grid((unsigned)l1_cdiv(T, 64), (unsigned)(B * n_hg), 1), block(64 * NH);
+	// the dA kernel takes up to eight heads per workgroup: longer runs of consecutive heads per store
+	const int NHa = (int)(H < DA_NH ? H : DA_NH);
+	const int64_t n_hga = l1_cdiv(H, NHa);
+	const dim3 grida((unsigned)l1_cdiv(T, 64), (unsigned)(B * n_hga), 1), blocka(64 * NHa);
 #define L1_FUSED_BWD_CASE(WV)                                                                                       \
 	case WV:                                                                                                        \
-		hipLaunchKernelGGL(fused_bwd_da_tile<WV>, grid, block, 0, st, dvo, q, k, v, vo, lse, dA, (int)T, (int)H,     \
-		                   (int)n_hg, NH, scale);                                                                   \
+		hipLaunchKernelGGL(fused_bwd_da_tile<WV>, grida, blocka, 0, st, dvo, q, k, v, vo, lse, dA, (int)T, (int)H,   \
+		                   (int)n_hga, NHa, scale);                                                                 \
 		hipLaunchKernelGGL(fused_bwd_dv_tile<WV>, grid, block, 0, st, dvo, q, k, lse, dv, (int)T, (int)H, (int)n_hg,  \
 		                   NH, scale);                                                                              \
 		break

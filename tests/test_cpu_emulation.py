@@ -26,8 +26,17 @@ EMU = os.path.join(HERE, "cpu_emu")
 @pytest.fixture(scope="module")
 def runner(tmp_path_factory):
     exe = str(tmp_path_factory.mktemp("emu") / "run_fused")
-    cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+    cmd = ["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
            "-I", EMU, "-x", "c++", os.path.join(EMU, "run_fused.cpp"), "-o", exe]
+    subprocess.run(cmd, check=True)
+    return exe
+
+
+@pytest.fixture(scope="module")
+def runner_tsan(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("emu_tsan") / "run_fused")
+    cmd = ["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=thread", "-I", EMU, "-x", "c++",
+           os.path.join(EMU, "run_fused.cpp"), "-o", exe]
     subprocess.run(cmd, check=True)
     return exe
 
@@ -92,7 +101,8 @@ TILED = [
     (2, 64, 4, 32),    # first baseline configuration
     (1, 100, 3, 64),   # ragged last dst tile, fewer heads than a workgroup holds
     (2, 70, 6, 16),    # ragged head group (4 + 2)
-    (3, 33, 9, 16),    # 27 workgroups: the XCD permutation leaves a remainder of three
+    (3, 33, 9, 16),    # 27 workgroups: the XCD permutation leaves a remainder of three; dA kernel: 8 + 1 heads
+    (1, 75, 16, 32),   # dA kernel: two full groups of eight heads; 75 = 9 flushes of 8 src rows + 3
 ]
 
 
@@ -102,9 +112,10 @@ def test_fused_tiled_kernels_on_cpu(runner, tmp_path, shape):
     g = torch.Generator().manual_seed(sum(shape))
     q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
     r = _run(runner, tmp_path, q, k, v)
-    NH = min(H, 4)
+    NH, NHa = min(H, 4), min(H, 8)  # heads per workgroup: forward and dv kernels, dA kernel
     launch = -(-T // 64) * B * -(-H // NH) * 64 * NH  # a tiled kernel's launch, not a generic one's
-    assert r["threads"] == launch and r["bwd_threads"] == 2 * launch
+    launch_a = -(-T // 64) * B * -(-H // NHa) * 64 * NHa
+    assert r["threads"] == launch and r["bwd_threads"] == launch + launch_a
     ref, ref_lse = _ref(q, k, v)
     assert cf.rel_err(r["vo"], ref) <= 1e-5 and cf.rel_err(r["lse"], ref_lse) <= 1e-5
     _check_backward(r, q, k, v, 1e-4)
@@ -141,4 +152,15 @@ def test_fused_unaligned_buffers_take_the_generic_kernels(runner, tmp_path):
     assert r["threads"] == B * T * H * W  # one thread per output element
     ref, ref_lse = _ref(q, k, v)
     assert cf.rel_err(r["vo"], ref) <= 1e-5 and cf.rel_err(r["lse"], ref_lse) <= 1e-5
+    _check_backward(r, q, k, v, 1e-4)
+
+
+def test_fused_kernels_have_no_data_race_between_barriers(runner_tsan, tmp_path):
+    """The same run under ThreadSanitizer (GPU threads are OS threads, __syncthreads() a barrier): the LDS tile of
+    the dA kernel is written and read by different threads, so a missing or misplaced barrier is a reported data
+    race and a non-zero exit (checked once by removing the barrier after the flush).  Ragged tile, 8 + 1 heads."""
+    B, T, H, W = 1, 75, 9, 16
+    g = torch.Generator().manual_seed(1)
+    q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
+    r = _run(runner_tsan, tmp_path, q, k, v)
     _check_backward(r, q, k, v, 1e-4)
