@@ -132,8 +132,8 @@ int l1attn_dense_column_ranks_f32(const float* q, const float* k, float* rq, flo
  * 32-bit integers on a common grid g = max(|q|,|k|) * 2^-24 (caller-owned workspace of
  * l1attn_dense_fwd_fixed_workspace_bytes), the pair-element is then one v_sad_u32 (|a-b|+c) instead of a
  * subtraction and an addition, the sum over W is exact, and attn = sum * g * (-1/sqrt(W)) in fp32.
- * Inputs and output are fp32 as in l1attn_dense_fwd_f32; each input is rounded to at most g/2, which is
- * the fp32 spacing of the head's largest values, so logits differ from the fp32 kernel's by about 1e-7 of
+ * Inputs and output are fp32 as in l1attn_dense_fwd_f32; each input moves by at most 0.75 g (g is between
+ * half and one fp32 spacing of the head's largest values), so logits differ from the fp32 kernel's by about 1e-7 of
  * the largest logit on N(0,1) or LayerNorm-scaled inputs (tolerance 1e-5).  Inputs must be finite.
  * Only W = 32 or 64, T >= 32, 16-byte aligned q and k (L1ATTN_ERR_ARG otherwise).  No counterpart in the
  * reference; not the default path of the Python operator.

@@ -164,3 +164,45 @@ def test_fused_kernels_have_no_data_race_between_barriers(runner_tsan, tmp_path)
     q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
     r = _run(runner_tsan, tmp_path, q, k, v)
     _check_backward(r, q, k, v, 1e-4)
+
+
+def test_fixed_point_prepass_kernels_on_cpu(tmp_path):
+    """The grid and conversion kernels of the experimental fixed-point forward (csrc/fixed.hip; one with an LDS
+    reduction) under AddressSanitizer: grids equal max(|q|,|k|) * 2^-24 per (batch, head) bit for bit, the
+    converted values equal rint(x / grid) with the sign bit flipped, bit for bit, and decode to within three quarters of a
+    grid step of the input; an all-zero head and a head 1000 times larger than the others."""
+    exe = str(tmp_path / "run_fixed")
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
+                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_fixed.cpp"), "-o", exe],
+                   check=True)
+    B, T, H, W = 2, 37, 3, 32
+    g = torch.Generator().manual_seed(11)
+    q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))
+    q[:, :, 1] *= 1000.0
+    q[1, :, 2] = 0
+    k[1, :, 2] = 0
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    with open(fin, "wb") as f:
+        f.write(struct.pack("4q", B, T, H, W))
+        f.write(q.numpy().tobytes())
+        f.write(k.numpy().tobytes())
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
+    r = subprocess.run([exe, fin, fout], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, (r.returncode, r.stderr[-2000:])
+    raw = open(fout, "rb").read()
+    n = B * T * H * W
+    gq = np.frombuffer(raw, np.float32, B * H).reshape(B, H)
+    uq = np.frombuffer(raw, np.uint32, n, B * H * 4).reshape(B, T, H, W)
+    uk = np.frombuffer(raw, np.uint32, n, B * H * 4 + n * 4).reshape(B, T, H, W)
+    qn, kn = q.numpy(), k.numpy()
+    m = np.maximum(np.abs(qn).max(axis=(1, 3)), np.abs(kn).max(axis=(1, 3)))            # [B,H]
+    g_ref = np.maximum(m * np.float32(2.0 ** -24), np.float32(1.17549435e-38)).astype(np.float32)
+    assert np.array_equal(gq, g_ref)
+    for x, u in ((qn, uq), (kn, uk)):
+        i_ref = np.rint((x / g_ref[:, None, :, None]).astype(np.float32)).astype(np.int64)
+        assert np.abs(i_ref).max() <= 2 ** 24
+        assert np.array_equal(u, ((i_ref + 2 ** 31) % 2 ** 32).astype(np.uint32))
+        decoded = (u.astype(np.int64) - 2 ** 31) * g_ref[:, None, :, None].astype(np.float64)
+        # half a step from rint, up to a quarter more from the fp32 rounding of the quotient below 2^23
+        assert np.all(np.abs(decoded - x) <= 0.7500001 * g_ref[:, None, :, None])
+    assert np.all(uq[1, :, 2] == 2 ** 31) and np.all(uk[1, :, 2] == 2 ** 31)
