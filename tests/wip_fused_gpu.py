@@ -212,3 +212,54 @@ def test_fixed_point_forward_vs_oracle(shape, layernorm):
     assert torch.count_nonzero(z[..., H - 1]) == 0 and torch.isfinite(z).all()
     with pytest.raises(RuntimeError, match="invalid argument"):
         drv.dense_forward_fixed(torch.zeros(1, 64, 2, 48).cuda(), torch.zeros(1, 64, 2, 48).cuda())
+
+
+@pytest.mark.parametrize("ntok", [21, 45])
+def test_fused_in_a_model_block(ntok):
+    """The reference's transformer block (example-setfind/setfind.py:98-138: q from a linear layer, k a gated
+    broadcast view of x, zero-token padding to a multiple of 16, one logit row overwritten with the no-op 0,
+    softmax over src, contraction with v, sum over heads) with the fused operator in place of its five steps
+    from the padding to the einsum: no padding is needed, the no-op is part of the operator.  Yardstick: the
+    reference's graph in fp64 with the closed form for the logits; gradients back to x and the weights.
+    21 tokens take the generic kernels, 45 the tiled ones."""
+    print("case fused model block", ntok, flush=True)
+    import math
+    fz = _fused()
+    batch, d_model, n_head = 3, 32, 4
+
+    def qkv(x, wq, wv, wk):
+        q = (x @ wq).reshape(batch, ntok, n_head, d_model)
+        v = (x @ wv).reshape(batch, ntok, n_head, d_model)
+        k = x.unsqueeze(2).expand(-1, -1, n_head, -1) * wk.unsqueeze(0).unsqueeze(0)
+        return q, k, v
+
+    def block_ref(x, wq, wv, wk):
+        q, k, v = qkv(x, wq, wv, wk)
+        padn = ((ntok + 15) // 16) * 16 - ntok
+        zeros = torch.zeros(batch, padn, n_head, d_model, dtype=x.dtype, device=x.device)
+        a = cf.dense_attn(torch.cat((q, zeros), 1), torch.cat((k, zeros), 1))
+        a = a[:, :ntok + 1, :ntok, :].clone()
+        a[:, ntok, :, :] = 0.0
+        a = torch.softmax(a, 1)[:, :ntok]
+        return torch.einsum("bsdh,bshw->bdhw", a, v).sum(2)
+
+    def block_fused(x, wq, wv, wk):
+        q, k, v = qkv(x, wq, wv, wk)
+        return fz.L1AttnFused()(q, k, v).sum(2)
+
+    def leaves(dtype):
+        g = torch.Generator().manual_seed(99)
+        x = torch.randn(batch, ntok, d_model, generator=g)
+        wq = torch.randn(d_model, n_head * d_model, generator=g) / math.sqrt(d_model)
+        wv = torch.randn(d_model, n_head * d_model, generator=g) / math.sqrt(d_model)
+        wk = torch.randn(n_head, d_model, generator=g)
+        return [t.to(dtype).cuda().requires_grad_() for t in (x, wq, wv, wk)]
+
+    got, ref = leaves(torch.float32), leaves(torch.float64)
+    out, out_ref = block_fused(*got), block_ref(*ref)
+    gout = torch.randn(out.shape, generator=torch.Generator().manual_seed(5)).cuda()
+    out.backward(gout)
+    out_ref.backward(gout.double())
+    assert cf.rel_err(out.detach().cpu(), out_ref.detach().cpu()) <= 1e-5
+    for a, b in zip(got, ref):
+        assert cf.rel_err(a.grad.cpu(), b.grad.cpu()) <= 1e-4
