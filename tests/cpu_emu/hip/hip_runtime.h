@@ -22,7 +22,14 @@
 #define __forceinline__ inline
 #define __launch_bounds__(...)
 #define __restrict__
+// Statically sized __shared__ arrays become static storage.  A source that only declares the dynamic array
+// (`extern __shared__ unsigned char name[];`) is built with EMU_DYNAMIC_LDS_ONLY: the declaration then names a
+// global array that the test driver defines.
+#ifdef EMU_DYNAMIC_LDS_ONLY
+#define __shared__
+#else
 #define __shared__ static
+#endif
 
 struct dim3 {
 	unsigned x, y, z;
@@ -30,6 +37,9 @@ struct dim3 {
 };
 struct float4 { float x, y, z, w; };
 static inline float4 make_float4(float x, float y, float z, float w) { return float4{x, y, z, w}; }
+struct double2 { double x, y; };
+static inline double2 make_double2(double x, double y) { return double2{x, y}; }
+struct uint2 { unsigned x, y; };
 
 typedef void* hipStream_t;
 typedef int hipError_t;
@@ -41,6 +51,12 @@ inline thread_local dim3 threadIdx_;
 inline dim3 blockIdx_, blockDim_, gridDim_;
 inline long n_threads_run = 0;
 inline std::unique_ptr<std::barrier<>> wg_barrier;  // the running workgroup's __syncthreads()
+// Lanes of a wavefront run in lockstep on the GPU; here they are OS threads, so every cross-lane exchange is
+// bracketed by a barrier among the wave's 64 threads.
+inline std::vector<std::unique_ptr<std::barrier<>>> wave_barrier;
+inline std::vector<double> wave_slots;  // 64 exchange slots per wave
+inline unsigned flat_tid() { return threadIdx_.x + blockDim_.x * (threadIdx_.y + blockDim_.y * threadIdx_.z); }
+inline void wave_sync() { wave_barrier[flat_tid() >> 6]->arrive_and_wait(); }
 }
 #define threadIdx (emu::threadIdx_)
 #define blockIdx (emu::blockIdx_)
@@ -52,6 +68,20 @@ using std::max;
 
 // value of the wave's first active lane; the kernels built here only pass wave-uniform values
 static inline int __builtin_amdgcn_readfirstlane(int x) { return x; }
+// Cross-lane read within the wave: every lane of the wave must call it (uniform control flow).
+template <typename T>
+static inline T __shfl_xor(T x, int lane_mask)
+{
+	const unsigned tid = emu::flat_tid(), base = tid & ~63u;
+	emu::wave_slots[tid] = (double)x;
+	emu::wave_sync();
+	const T r = (T)emu::wave_slots[base + ((tid ^ (unsigned)lane_mask) & 63u)];
+	emu::wave_sync();
+	return r;
+}
+// Memory fences order a wave's own stores before its own later loads from other lanes: lockstep lanes need
+// nothing more on the GPU, OS threads need a barrier among the wave.
+#define __builtin_amdgcn_fence(order, scope) emu::wave_sync()
 // every thread of the workgroup must reach it (a thread that has returned would hang the others, as it may on a GPU)
 static inline void __syncthreads() { emu::wg_barrier->arrive_and_wait(); }
 
@@ -69,6 +99,10 @@ static inline void emu_launch(K kernel, dim3 grid, dim3 block, A... args)
 			if (tid == 0) {
 				emu::blockIdx_ = dim3((unsigned)(bi % grid.x), (unsigned)((bi / grid.x) % grid.y), (unsigned)(bi / ((long)grid.x * grid.y)));
 				emu::wg_barrier.reset(new std::barrier<>(nt));
+				emu::wave_barrier.clear();
+				for (unsigned w = 0; w < (nt + 63) / 64; w++)
+					emu::wave_barrier.emplace_back(new std::barrier<>(std::min(64u, nt - w * 64)));
+				emu::wave_slots.assign((nt + 63) / 64 * 64, 0.0);
 			}
 			step.arrive_and_wait();
 			kernel(args...);
