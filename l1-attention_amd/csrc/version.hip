@@ -1,7 +1,7 @@
 // Library identification, and a probe of what the fp32 VALU of this GPU gives to ordinary code.
 #include "common.h"
 
-extern "C" int l1attn_version(void) { return 100; }
+extern "C" int l1attn_version(void) { return 10100; }  // 1.1.0: fused operator, 16-bit sparse forwards, probes
 
 namespace {
 
