@@ -153,7 +153,7 @@ int l1attn_dense_fwd_fixed_f32(const float* q, const float* k, float* attn,
  * l1attn_cuda_drv.forward (a zero logit row appended, softmax over dim 1, 'bsdh,bshw->bdhw':
  * example-setfind/setfind.py:128-136, python/l1attn_sparse.py:488-506) and the form its README asks
  * for (README.md:21).  q,k [B,T,H,W]; v,vo [B,T,H,Wv].  Deterministic.  Backward: below.
- * f32: W == Wv in {16,32,64}, T >= 32 and 16-byte aligned pointers run the tiled kernel; every other
+ * f32: W == Wv in {16,32,48,64,96}, T >= 32 and 16-byte aligned pointers run the tiled kernel; every other
  * shape, and f64, a generic one (L1ATTN_ERR_RANGE when it would need 2^32 threads or more).
  */
 int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse,

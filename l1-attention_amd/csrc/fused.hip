@@ -26,8 +26,10 @@ template <typename T> __device__ __forceinline__ T fabs_t(T x) { return x < (T)0
 template <typename T> __device__ __forceinline__ T exp_t(T x);
 template <> __device__ __forceinline__ float exp_t<float>(float x) { return expf(x); }
 template <> __device__ __forceinline__ double exp_t<double>(double x) { return exp(x); }
-__device__ __forceinline__ float log_t(float x) { return logf(x); }
-__device__ __forceinline__ double log_t(double x) { return log(x); }
+// log(1 + x): the sum of the weights is often far below 1 (long L1 distances), where log(1 + x) formed in two
+// steps would lose most of its digits
+__device__ __forceinline__ float log1p_t(float x) { return log1pf(x); }
+__device__ __forceinline__ double log1p_t(double x) { return log1p(x); }
 
 // Any shape, float or double: one thread per output element (b,t,h,wv); the logit of each src token is
 // recomputed by every thread of the row (W-fold redundant), which only small or odd shapes pay.
@@ -50,13 +52,13 @@ __global__ __launch_bounds__(256) void fused_fwd_generic(const T* __restrict__ q
 		den += p;
 		acc += p * v[((b * Tn + s) * H + h) * Wv + wv];
 	}
-	den += (T)1;
-	vo[idx] = acc / den;
-	if (lse && wv == 0) lse[(b * Tn + t) * H + h] = log_t(den);
+	vo[idx] = acc / ((T)1 + den);
+	if (lse && wv == 0) lse[(b * Tn + t) * H + h] = log1p_t(den);
 }
 
 // grid.x = dst tiles of 64 tokens, grid.y = B * head groups; block = 64 * NH threads, wave w owns head
-// hg*NH + w.  W == WV is a compile-time multiple of 16; q, k, v, vo must be 16-byte aligned.
+// hg*NH + w.  W == WV is a compile-time multiple of 16 (16, 32, 48, 64, 96: q and the output row must fit the
+// registers); q, k, v, vo must be 16-byte aligned.
 template <int W>
 __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ vo,
@@ -99,15 +101,14 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restric
 		kp += row;
 		vp += row;
 	}
-	den += 1.0f;
 	if (store) {
-		const float inv = 1.0f / den;
+		const float inv = 1.0f / (1.0f + den);
 		float4* op = reinterpret_cast<float4*>(vo + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
 #pragma unroll
 		for (int w4 = 0; w4 < W / 4; w4++)
 			op[w4] = make_float4(acc[w4 * 4 + 0] * inv, acc[w4 * 4 + 1] * inv, acc[w4 * 4 + 2] * inv,
 			                     acc[w4 * 4 + 3] * inv);
-		if (lse) lse[((int64_t)b * Tn + t) * H + h] = logf(den);
+		if (lse) lse[((int64_t)b * Tn + t) * H + h] = log1pf(den);
 	}
 }
 
@@ -335,7 +336,7 @@ int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* 
 	const bool aligned = ((((uintptr_t)q) | ((uintptr_t)k) | ((uintptr_t)v) | ((uintptr_t)vo)) & 15) == 0;
 	const int NH = (int)(H < 4 ? H : 4);
 	const int64_t n_hg = l1_cdiv(H, NH);
-	const bool tiled = aligned && W == Wv && (W == 16 || W == 32 || W == 64) && T >= 32 && T <= (1 << 30) &&
+	const bool tiled = aligned && W == Wv && (W == 16 || W == 32 || W == 48 || W == 64 || W == 96) && T >= 32 && T <= (1 << 30) &&
 	                   B * n_hg <= 65535 && H <= 65535;
 	if (!tiled) return launch_generic<float>(q, k, v, vo, lse, B, T, H, W, Wv, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
@@ -348,7 +349,9 @@ int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* 
 	switch (W) {
 		L1_FUSED_CASE(16);
 		L1_FUSED_CASE(32);
+		L1_FUSED_CASE(48);
 		L1_FUSED_CASE(64);
+		L1_FUSED_CASE(96);
 	default: return L1ATTN_ERR_ARG;
 	}
 #undef L1_FUSED_CASE
@@ -379,7 +382,7 @@ int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k,
 	                       ((uintptr_t)dv)) & 15) == 0;
 	const int NH = (int)(H < 4 ? H : 4);
 	const int64_t n_hg = l1_cdiv(H, NH);
-	const bool tiled = aligned && W == Wv && (W == 16 || W == 32 || W == 64) && T >= 32 && T <= (1 << 30) &&
+	const bool tiled = aligned && W == Wv && (W == 16 || W == 32 || W == 48 || W == 64 || W == 96) && T >= 32 && T <= (1 << 30) &&
 	                   B * n_hg <= 65535 && H <= 65535;
 	if (!tiled) return launch_bwd_generic<float>(dvo, q, k, v, vo, lse, dA, dv, B, T, H, W, Wv, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
@@ -398,7 +401,9 @@ int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k,
 	switch (W) {
 		L1_FUSED_BWD_CASE(16);
 		L1_FUSED_BWD_CASE(32);
+		L1_FUSED_BWD_CASE(48);
 		L1_FUSED_BWD_CASE(64);
+		L1_FUSED_BWD_CASE(96);
 	default: return L1ATTN_ERR_ARG;
 	}
 #undef L1_FUSED_BWD_CASE

@@ -103,6 +103,7 @@ TILED = [
     (2, 70, 6, 16),    # ragged head group (4 + 2)
     (3, 33, 9, 16),    # 27 workgroups: the XCD permutation leaves a remainder of three; dA kernel: 8 + 1 heads
     (1, 75, 16, 32),   # dA kernel: two full groups of eight heads; 75 = 9 flushes of 8 src rows + 3
+    (1, 40, 2, 48), (1, 36, 5, 96),  # the other two tiled widths
 ]
 
 
@@ -123,7 +124,7 @@ def test_fused_tiled_kernels_on_cpu(runner, tmp_path, shape):
 
 GENERIC = [
     # B, T, H, W, Wv
-    (2, 3, 16, 7, 7), (1, 40, 2, 48, 48), (1, 37, 3, 32, 20), (1, 31, 2, 64, 64), (1, 1, 1, 1, 1),
+    (2, 3, 16, 7, 7), (1, 40, 2, 80, 80), (1, 37, 3, 32, 20), (1, 31, 2, 64, 64), (1, 1, 1, 1, 1),
 ]
 
 

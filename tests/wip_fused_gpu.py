@@ -37,7 +37,9 @@ SHAPES = [
     (2, 70, 6, 16, 16),     # tiled kernel, width 16, ragged head group (6 = 4 + 2)
     (1, 33, 9, 64, 64),     # three head groups, the last with one head
     (2, 3, 16, 7, 7),       # generic kernel (check_sparse.py:18-21 shape)
-    (1, 40, 2, 48, 48),     # generic kernel: width not among the tiled ones
+    (1, 40, 2, 48, 48),     # tiled kernel, width 48
+    (1, 36, 5, 96, 96),     # tiled kernel, width 96 (249-255 VGPRs)
+    (1, 40, 2, 80, 80),     # generic kernel: width not among the tiled ones
     (1, 37, 3, 32, 20),     # generic kernel: value width differs
     (1, 31, 2, 64, 64),     # generic kernel: fewer than 32 tokens
 ]
@@ -118,6 +120,7 @@ BWD_SHAPES = [
     (2, 64, 4, 32, 32),     # tiled kernels
     (1, 100, 3, 64, 64),    # tiled, ragged tile, 164 and 167 VGPR instantiations
     (2, 70, 6, 16, 16),     # tiled, ragged head group
+    (1, 40, 2, 48, 48), (1, 36, 5, 96, 96),  # the other two tiled widths
     (2, 9, 3, 5, 5),        # generic kernels
     (1, 37, 3, 32, 20),     # generic kernels, value width differs
 ]
