@@ -26,9 +26,40 @@ static S* to_storage(const std::vector<float>& x)
 	return p;
 }
 
+template <typename S>
+static int backward(const int64_t*, const void*, const S*, const S*, const S*, const S*, const S*, const S*, FILE*)
+{
+	return 0;  // the 16-bit types have no backward
+}
+#define L1_EMU_BWD(SFX, TYPE)                                                                                       \
+	template <>                                                                                                     \
+	int backward<TYPE>(const int64_t* d, const void* plan, const TYPE* dvo, const TYPE* vf, const TYPE* vb,         \
+	                   const TYPE* q, const TYPE* k, const TYPE* P, FILE* fo)                                       \
+	{                                                                                                               \
+		const int64_t B = d[0], T = d[1], H = d[2], W = d[3], Wv = d[4], E = d[5];                                  \
+		const size_t nv = (size_t)(B * T * H * Wv), nq = (size_t)(B * T * H * W), ne = (size_t)(B * E * H);         \
+		auto al = [](size_t n) { return (TYPE*)aligned_alloc(16, (n * sizeof(TYPE) + 15) / 16 * 16 + 16); };        \
+		TYPE *dvf = al(nv), *dvb = al(nv), *dq = al(nq), *dk = al(nq), *DA = al(ne);                                \
+		for (size_t i = 0; i < nv; i++) dvb[i] = 0;                                                                 \
+		const int rc = d[7] ? l1attn_sparse_bidi_bwd_##SFX(dvo, vf, vb, q, k, plan, P, dvf, dvb, dq, dk, DA, B, T,  \
+		                                                   H, W, Wv, E, (int)d[6], nullptr)                         \
+		                    : l1attn_sparse_bwd_##SFX(dvo, vf, q, k, plan, P, dvf, dq, dk, DA, B, T, H, W, Wv, E,    \
+		                                              (int)d[6], nullptr);                                          \
+		if (rc) return 30 + (rc < 0 ? -rc : rc);                                                                    \
+		for (size_t i = 0; i < nv; i++) { const double x = (double)dvf[i]; fwrite(&x, 8, 1, fo); }                  \
+		for (size_t i = 0; i < nv; i++) { const double x = (double)dvb[i]; fwrite(&x, 8, 1, fo); }                  \
+		for (size_t i = 0; i < nq; i++) { const double x = (double)dq[i]; fwrite(&x, 8, 1, fo); }                   \
+		for (size_t i = 0; i < nq; i++) { const double x = (double)dk[i]; fwrite(&x, 8, 1, fo); }                   \
+		free(dvf); free(dvb); free(dq); free(dk); free(DA);                                                         \
+		return 0;                                                                                                   \
+	}
+L1_EMU_BWD(f32, float)
+L1_EMU_BWD(f64, double)
+
 template <typename S, typename P, typename F>
 static int run(const int64_t* d, const void* plan, const std::vector<float>& vf, const std::vector<float>& vb,
-               const std::vector<float>& q, const std::vector<float>& k, FILE* fo, F call)
+               const std::vector<float>& q, const std::vector<float>& k, const std::vector<float>& dvo, FILE* fo,
+               F call)
 {
 	const int64_t B = d[0], T = d[1], H = d[2], Wv = d[4], E = d[5];
 	S *pvf = to_storage<S>(vf), *pvb = to_storage<S>(vb), *pq = to_storage<S>(q), *pk = to_storage<S>(k);
@@ -38,6 +69,12 @@ static int run(const int64_t* d, const void* plan, const std::vector<float>& vf,
 	if (rc) return 10 + (rc < 0 ? -rc : rc);
 	for (int64_t i = 0; i < B * T * H * Wv; i++) { const double x = (double)vo[i]; fwrite(&x, 8, 1, fo); }
 	for (int64_t i = 0; i < B * E * H; i++) { const double x = (double)pw[i]; fwrite(&x, 8, 1, fo); }
+	if (sizeof(S) == sizeof(P)) {  // float32 / float64: the backward on the weights just written
+		S* pdvo = to_storage<S>(dvo);
+		const int rcb = backward<S>(d, plan, pdvo, pvf, pvb, pq, pk, (const S*)pw, fo);
+		free(pdvo);
+		if (rcb) return rcb;
+	}
 	free(pvf); free(pvb); free(pq); free(pk); free(vo); free(pw);
 	return 0;
 }
@@ -60,12 +97,12 @@ int main(int argc, char** argv)
 	if (!rd(L.dst_ptr, T + 2) || !rd(L.src_ptr, T + 2) || !rd(L.csr_src, E) || !rd(L.csr_row, E) || !rd(L.csc_dst, E) ||
 	    !rd(L.csc_slot, E) || !rd(L.long_dst, d[9]) || !rd(L.long_src, d[10]))
 		return 3;
-	std::vector<float> vf(B * T * H * Wv), vb(B * T * H * Wv), q(B * T * H * W), k(B * T * H * W);
-	for (auto* x : {&vf, &vb, &q, &k})
+	std::vector<float> vf(B * T * H * Wv), vb(B * T * H * Wv), q(B * T * H * W), k(B * T * H * W), dvo(B * T * H * Wv);
+	for (auto* x : {&vf, &vb, &q, &k, &dvo})
 		if (fread(x->data(), 4, x->size(), fi) != x->size()) return 3;
 	int rc;
 #define CALL(SFX, S, P)                                                                                              \
-	rc = run<S, P>(d, plan.data(), vf, vb, q, k, fo,                                                                 \
+	rc = run<S, P>(d, plan.data(), vf, vb, q, k, dvo, fo,                                                               \
 	               [&](const S* a, const S* b, const S* qq, const S* kk, const void* pl, S* vo, P* pw) {             \
 		               return bidi ? l1attn_sparse_bidi_fwd_##SFX(a, b, qq, kk, pl, vo, pw, B, T, H, W, Wv, E, sm, nullptr) \
 		                           : l1attn_sparse_fwd_##SFX(a, qq, kk, pl, vo, pw, B, T, H, W, Wv, E, sm, nullptr);  \

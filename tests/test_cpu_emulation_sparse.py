@@ -1,6 +1,7 @@
-"""CPU run of the sparse and bidirectional forward kernels (csrc/sparse.hip compiled for the host against
+"""CPU run of the sparse and bidirectional kernels, forward and backward (csrc/sparse.hip compiled for the host against
 tests/cpu_emu/hip/hip_runtime.h: GPU threads are OS threads, cross-lane reads, fences and __syncthreads() are
-barriers) under AddressSanitizer, for float32, float64, float16 and bfloat16 rows, against the oracle.
+barriers) under AddressSanitizer, for float32, float64 and (forward) float16 and bfloat16 rows, against fp64
+closed forms and torch autograd through them.
 
 It covers what the 16-bit entry points add to kernels that the GPU tests already cover in float32 and float64:
 conversion on load, rounding on store, 8-byte row pieces, and the claim their GPU test rests on -- that the
@@ -69,7 +70,8 @@ def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind):
         f.write(struct.pack("11q", B, T, H, W, Wv, E, int(sm), int(bidi), TYPES[kind], len(arrays[6]), len(arrays[7])))
         for a in arrays:
             f.write(a.tobytes())
-        for x in (vf, vb, q, k):
+        dvo = torch.randn(B, T, H, Wv, generator=torch.Generator().manual_seed(77))
+        for x in (vf, vb, q, k, dvo):
             f.write(x.float().contiguous().numpy().tobytes())
     env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
     r = subprocess.run([exe, fin, fout], env=env, capture_output=True, text=True)
@@ -77,9 +79,30 @@ def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind):
     raw = np.fromfile(fout, np.float64)
     nv = B * T * H * Wv
     vo = torch.from_numpy(raw[:nv].copy()).view(B, T, H, Wv)
-    P = torch.from_numpy(raw[nv:].copy()).view(B, E, H)
+    P = torch.from_numpy(raw[nv:nv + B * E * H].copy()).view(B, E, H)
     slot_row = torch.from_numpy(arrays[3].astype(np.int64))  # original row of each slot
+    _run.grads = None
+    if kind in ("f32", "f64"):  # the driver also ran the backward on dvo
+        pos, nq = nv + B * E * H, B * T * H * W
+        take = lambda n, shape: torch.from_numpy(raw[pos:pos + n].copy()).view(*shape)
+        dvf = take(nv, (B, T, H, Wv)); pos += nv
+        dvb = take(nv, (B, T, H, Wv)); pos += nv
+        dq = take(nq, (B, T, H, W)); pos += nq
+        dk = take(nq, (B, T, H, W)); pos += nq
+        assert pos == raw.shape[0]
+        _run.grads = (dvo.double(), dvf, dvb, dq, dk)
     return vo, P, slot_row
+
+
+def _check_grads(vf, vb, q, k, co, sm, bidi, tol):
+    """The backward the last _run performed, against torch autograd through the fp64 closed form."""
+    dvo, dvf, dvb, dq, dk = _run.grads
+    x = [t.double().requires_grad_() for t in (vf, vb, q, k)]
+    out = cf.bidi_value(x[0], x[1], x[2], x[3], co, sm) if bidi else cf.sparse_value(x[0], x[2], x[3], co, sm)
+    ref = torch.autograd.grad(out, x, dvo, allow_unused=True)
+    assert cf.rel_err(dvf, ref[0]) <= tol and cf.rel_err(dq, ref[2]) <= tol and cf.rel_err(dk, ref[3]) <= tol
+    if bidi:
+        assert cf.rel_err(dvb, ref[1]) <= tol
 
 
 TOL = {"f16": 2.0 ** -10, "bf16": 2.0 ** -7}
@@ -104,6 +127,7 @@ def test_sparse_forward_kernels_on_cpu(runner, tmp_path, shape, sm):
         assert cf.rel_err(vo32, ref) <= 1e-5
         p_ref = cf.edge_probs(q.double(), k.double(), co, sm)[:, slot_row]  # weights in slot order
         assert cf.rel_err(P32, p_ref) <= 1e-5
+        _check_grads(vf, vb, q, k, co, sm, False, 1e-4)
         vo16, P16, _ = _run(runner, tmp_path, vf, vb, q, k, co, sm, False, kind)
         assert torch.equal(P16, P32)
         assert torch.equal(vo16.float(), vo32.float().to(dt).float())
@@ -111,6 +135,13 @@ def test_sparse_forward_kernels_on_cpu(runner, tmp_path, shape, sm):
         vob, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, sm, True, kind)
         ref = cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, sm)
         assert cf.rel_err(vob, ref) <= TOL[kind]
+    # float64, both operators, forward and backward
+    for bidi in (False, True):
+        vo, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, sm, bidi, "f64")
+        ref = cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, sm) if bidi else \
+            cf.sparse_value(vf.double(), q.double(), k.double(), co, sm)
+        assert cf.rel_err(vo, ref) <= 1e-12
+        _check_grads(vf, vb, q, k, co, sm, bidi, 1e-11)
 
 
 def test_sparse_forward_long_segment_on_cpu(runner, tmp_path):
@@ -130,3 +161,6 @@ def test_sparse_forward_long_segment_on_cpu(runner, tmp_path):
     assert torch.equal(P16, P32) and torch.equal(vo16.float(), vo32.float().half().float())
     vob, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, True, True, "f16")
     assert cf.rel_err(vob, cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, True)) <= TOL["f16"]
+    vob, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, True, True, "f32")
+    assert cf.rel_err(vob, cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, True)) <= 1e-5
+    _check_grads(vf, vb, q, k, co, True, True, 1e-4)  # long segments in both backward passes
