@@ -4,7 +4,9 @@
 // __syncthreads() is a barrier among them, __shared__ arrays are static storage (workgroups run one
 // after the other).  It checks a kernel's index arithmetic, clamps, store predicates, LDS indexing,
 // barrier placement and launch geometry against exactly-sized host buffers; it says nothing about
-// timing, the memory model or the hardware.  Never part of the library: only
+// timing, the memory model or the hardware.  Lanes of a wave do not run in lockstep here: a kernel
+// whose lanes hand values to each other through memory without a fence or a cross-lane operation in
+// between (the radix sort of coo.hip does, through per-wave LDS counters) cannot be run this way.  Never part of the library: only
 // tests/test_cpu_emulation.py builds with it.
 #pragma once
 #include <math.h>

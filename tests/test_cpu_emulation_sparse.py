@@ -164,3 +164,4 @@ def test_sparse_forward_long_segment_on_cpu(runner, tmp_path):
     vob, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, True, True, "f32")
     assert cf.rel_err(vob, cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, True)) <= 1e-5
     _check_grads(vf, vb, q, k, co, True, True, 1e-4)  # long segments in both backward passes
+
