@@ -95,6 +95,21 @@ def fused_fwd(q, k, v):
     return torch.einsum("bsdh,bshw->bdhw", p, v), torch.logsumexp(a, 1)
 
 
+def fused_bwd(dvo, q, k, v):
+    """Backward of fused_fwd along the reference's own pieces: the softmax and einsum steps of
+    example-setfind/setfind.py:128-136 differentiated by hand (softmax over src with the no-op row:
+    dA = P * (dP - sum_s P * dP), the no-op row's share dropped with the row), then dq, dk from the reference's
+    dense backward loop (cpp/l1attn_drv.cpp:57-98).  -> (dq, dk, dv)."""
+    B, T, H, W = q.shape
+    a = dense_fwd(q, k)
+    a = torch.cat((a, torch.zeros(B, 1, T, H, dtype=a.dtype)), 1)
+    p = torch.softmax(a, 1)[:, :T]                                   # [B,S,T,H]
+    dp = torch.einsum("bdhw,bshw->bsdh", dvo, v)
+    d_attn = p * (dp - (p * dp).sum(1, keepdim=True))
+    dq, dk = dense_bwd(d_attn.contiguous(), q, k)
+    return dq, dk, torch.einsum("bsdh,bdhw->bshw", p, dvo)
+
+
 def _coo32(coo):
     coo = coo.to(torch.int32).contiguous()
     assert coo.dim() == 2 and coo.shape[1] >= 3

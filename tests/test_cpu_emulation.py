@@ -94,6 +94,9 @@ def _check_backward(r, q, k, v, tol):
     dq_ref, dk_ref = torch.autograd.grad(cf.dense_then_value(qd, kd, v, noop=True), (qd, kd), dvo)
     dq, dk = oracle.dense_bwd(r["dA"].double(), q, k)
     assert cf.rel_err(dq, dq_ref) <= tol and cf.rel_err(dk, dk_ref) <= tol
+    if q.shape[3] == v.shape[3]:  # and the oracle's own backward agrees with autograd
+        odq, odk, odv = oracle.fused_bwd(dvo, q, k, v)
+        assert cf.rel_err(odq, dq_ref) <= 1e-11 and cf.rel_err(odk, dk_ref) <= 1e-11 and cf.rel_err(odv, dv_ref) <= 1e-11
 
 
 TILED = [

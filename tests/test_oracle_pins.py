@@ -248,6 +248,33 @@ def test_fused_forward_oracle_pins():
         assert abs(float(lse[b, t, h]) - math.log(1.0 + sum(e))) < 1e-13
 
 
+def test_fused_backward_oracle_pins():
+    """oracle.fused_bwd (hand-differentiated softmax and einsum, then the reference's dense backward loop) against
+    torch autograd through the broadcast closed form, against the sparse oracle's backward over the full cartesian
+    list (pinned by the reference extension's golden vectors), and by finite differences on one element each."""
+    g = torch.Generator().manual_seed(21)
+    B, T, H, W = 2, 6, 3, 4
+    q, k, v, dvo = (torch.randn(B, T, H, W, generator=g, dtype=torch.float64) for _ in range(4))
+    dq, dk, dv = oracle.fused_bwd(dvo, q, k, v)
+    x = [t.clone().requires_grad_() for t in (q, k, v)]
+    ref = torch.autograd.grad(cf.dense_then_value(*x, noop=True), x, dvo)
+    for a, b in zip((dq, dk, dv), ref):
+        assert torch.allclose(a, b, rtol=1e-12, atol=1e-13)
+    coo, dmx, _ = oracle.expand_coo(torch.cartesian_prod(torch.arange(T), torch.arange(T)))
+    _, attn = oracle.sparse_fwd(v, q, k, coo, dmx, True)
+    sdv, sdq, sdk = oracle.sparse_bwd(dvo, v, q, k, coo, attn, dmx, True, 0)
+    for a, b in zip((dq, dk, dv), (sdq, sdk, sdv)):
+        assert torch.allclose(a, b, rtol=1e-11, atol=1e-12)
+    loss = lambda q_, k_, v_: float((oracle.fused_fwd(q_, k_, v_)[0] * dvo).sum())
+    eps = 1e-6
+    for which, grad in ((0, dq), (1, dk), (2, dv)):
+        args = [q.clone(), k.clone(), v.clone()]
+        args[which][1, 2, 1, 3] += eps
+        up = loss(*args)
+        args[which][1, 2, 1, 3] -= 2 * eps
+        assert abs((up - loss(*args)) / (2 * eps) - float(grad[1, 2, 1, 3])) < 1e-7
+
+
 def test_sparse_integer_fixture_hand_answer():
     # python/l1attn_sparse.py:484 : co = [[0,0],[0,1],[1,0],[1,1],[2,2]], softmax on.
     # dst 0 sees k0 (L1=4) and k1 (L1=0): e = exp(-4/sqrt3), 1 ; denominator 1 + e + 1.
