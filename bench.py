@@ -171,15 +171,15 @@ def extra_legs():
     """Opt-in (--extra): the two additions beyond the reference's operators, timed beside what they replace.
     Fused forward (logits, softmax over src with the no-op logit, value sum in one kernel) against the same
     result composed from L1Attn and torch's cat / softmax / einsum, at the second baseline configuration and
-    the headline shape; sparse and bidirectional forwards with float16 / bfloat16 rows against float32 rows at
-    configurations 4 and 5.  Prints its own JSON line; the default run does not come here."""
+    the headline shape; sparse and bidirectional operators with float16 / bfloat16 rows against float32 rows at
+    configurations 4 and 5 (forward, and forward + backward).  Prints its own JSON line; the default run does not come here."""
     import torch
     import workloads
     import l1attn_cuda
     import l1attn_sparse_cuda as sp
     import l1attn_sparse_bidi_cuda as bi
     dev = torch.device("cuda:0")
-    res = {"fused_forward": {}, "sparse_forward_16bit": {}}
+    res = {"fused_forward": {}, "sparse_16bit": {}}
     for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
         q, k, v = (x.to(dev) for x in workloads.dense_inputs(B, T, H, W, seed=1002, with_v=True))
         fused, plain = l1attn_cuda.L1AttnFused(), l1attn_cuda.L1Attn()
@@ -239,8 +239,18 @@ def extra_legs():
         for dt in (torch.float32, torch.float16, torch.bfloat16):
             x = [t.to(dt) for t in x32]
             args = (x[0], x[1], x[2], x[3]) if bidi else (x[0], x[2], x[3])
-            row[str(dt).split(".")[1] + "_fwd_ms"] = time_gpu(lambda: m(*args, coo, dmx), 10)
-        res["sparse_forward_16bit"][name] = row
+            name_dt = str(dt).split(".")[1]
+            row[name_dt + "_fwd_ms"] = time_gpu(lambda: m(*args, coo, dmx), 10)
+            leaves = [t.clone().requires_grad_() for t in args]
+            dvo = torch.randn(B, T, H, W, device=dev).to(dt)
+
+            def fwdbwd():
+                for t in leaves:
+                    t.grad = None
+                m(*leaves, coo, dmx).backward(dvo)
+
+            row[name_dt + "_fwd_bwd_ms"] = time_gpu(fwdbwd, 10)
+        res["sparse_16bit"][name] = row
         log(name, json.dumps(row))
     import _l1attn_hip as drv
     res["fixed_point_forward"] = {}

@@ -298,9 +298,8 @@ int l1attn_sparse_bidi_bwd_f64(const double* dvo, const double* vf, const double
  * entry points; 16-byte aligned pointers with W and Wv multiples of 4 take the vector path.
  * Replaces the Half instantiation of the reference's forward launchers
  * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, cuda/l1attn_sparse_cuda_kernel.cu:405-435 and :684-714),
- * which computes every step in half precision.  There is no 16-bit backward, as in the reference:
- * its backward launchers dispatch float and double only (:483-519, :765-803).  bfloat16 is an
- * addition.
+ * which computes every step in half precision.  bfloat16 is an addition, and so are the 16-bit
+ * backwards below.
  */
 int l1attn_sparse_fwd_f16(const void* v, const void* q, const void* k, const void* plan,
                           void* vo, float* P,
@@ -316,6 +315,32 @@ int l1attn_sparse_bidi_fwd_f16(const void* vf, const void* vb, const void* q, co
                                int use_softmax, void* stream);
 int l1attn_sparse_bidi_fwd_bf16(const void* vf, const void* vb, const void* q, const void* k,
                                 const void* plan, void* vo, float* P,
+                                int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                                int use_softmax, void* stream);
+
+/*
+ * The two backwards with 16-bit rows: dvo, v/vf, vb, q, k and the gradients are binary16 or bfloat16 in
+ * memory; P (from the 16-bit forward) and the scratch DA are fp32, every sum runs in fp32, each gradient
+ * element is rounded to nearest even once on store.  No counterpart in the reference, whose backward
+ * launchers dispatch float and double only (cuda/l1attn_sparse_cuda_kernel.cu:483-519, :765-803); for
+ * mixed-precision training on the gather-bound path (six of the eight row gathers per edge are here).
+ */
+int l1attn_sparse_bwd_f16(const void* dvo, const void* v, const void* q, const void* k, const void* plan,
+                          const float* P, void* dv, void* dq, void* dk, float* DA,
+                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                          int use_softmax, void* stream);
+int l1attn_sparse_bwd_bf16(const void* dvo, const void* v, const void* q, const void* k, const void* plan,
+                           const float* P, void* dv, void* dq, void* dk, float* DA,
+                           int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                           int use_softmax, void* stream);
+int l1attn_sparse_bidi_bwd_f16(const void* dvo, const void* vf, const void* vb, const void* q, const void* k,
+                               const void* plan, const float* P,
+                               void* dvf, void* dvb, void* dq, void* dk, float* DA,
+                               int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
+                               int use_softmax, void* stream);
+int l1attn_sparse_bidi_bwd_bf16(const void* dvo, const void* vf, const void* vb, const void* q, const void* k,
+                                const void* plan, const float* P,
+                                void* dvf, void* dvb, void* dq, void* dk, float* DA,
                                 int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
                                 int use_softmax, void* stream);
 

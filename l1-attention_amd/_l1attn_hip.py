@@ -87,8 +87,9 @@ def lib():
                 f = getattr(L, name + sfx)
                 f.restype = _c_i
                 f.argtypes = [_c_p] * nptr + dims
-        for sfx in ("f16", "bf16"):  # forward only, as in the reference
-            for name, nptr in (("l1attn_sparse_fwd_", 6), ("l1attn_sparse_bidi_fwd_", 7)):
+        for sfx in ("f16", "bf16"):  # 16-bit rows, fp32 sums and edge weights
+            for name, nptr in (("l1attn_sparse_fwd_", 6), ("l1attn_sparse_bidi_fwd_", 7),
+                               ("l1attn_sparse_bwd_", 10), ("l1attn_sparse_bidi_bwd_", 12)):
                 f = getattr(L, name + sfx)
                 f.restype = _c_i
                 f.argtypes = [_c_p] * nptr + dims
@@ -121,9 +122,9 @@ def sfx_of(x, name="q"):
 
 
 def sfx_fwd_sparse(x, name="q"):
-    """Entry-point suffix and edge-weight dtype of the sparse forwards.  They also take 16-bit rows
-    (the reference dispatches Half there: cuda/l1attn_sparse_cuda_kernel.cu:405-435, :684-714);
-    the weights of a 16-bit forward are fp32."""
+    """Entry-point suffix and edge-weight dtype of the sparse operators.  They also take 16-bit rows
+    (the reference dispatches Half in its forwards: cuda/l1attn_sparse_cuda_kernel.cu:405-435, :684-714);
+    the weights of a 16-bit call are fp32."""
     if x.dtype == torch.float16:
         return "f16", torch.float32
     if x.dtype == torch.bfloat16:
@@ -132,12 +133,10 @@ def sfx_fwd_sparse(x, name="q"):
 
 
 def sfx_bwd_sparse(x):
-    """The sparse backwards exist for float32 and float64 only, like the reference's
-    (AT_DISPATCH_FLOATING_TYPES, cuda/l1attn_sparse_cuda_kernel.cu:483-519, :765-803)."""
-    if x.dtype in (torch.float16, torch.bfloat16):
-        raise RuntimeError("the sparse backward is not implemented for %s (forward only, as in the reference)"
-                           % x.dtype)
-    return sfx_of(x)
+    """Entry-point suffix of the sparse backwards.  The reference's exist for float32 and float64 only
+    (AT_DISPATCH_FLOATING_TYPES, cuda/l1attn_sparse_cuda_kernel.cu:483-519, :765-803); the 16-bit ones here are
+    an addition: gradients in the rows' type, sums and edge weights in fp32."""
+    return sfx_fwd_sparse(x)[0]
 
 
 def stream_of(x):
@@ -358,7 +357,8 @@ def _edge_tensors(coo, P, q, E, B, H):
     """coo (and the saved edge weights P, if given) must live on q's device; P is [batch, edges, heads]."""
     if coo.device != q.device:
         raise RuntimeError("coo must be on the device of q")
-    if P is not None and (tuple(P.shape) != (B, E, H) or P.dtype != q.dtype or P.device != q.device):
+    p_dtype = torch.float32 if q.dtype in (torch.float16, torch.bfloat16) else q.dtype
+    if P is not None and (tuple(P.shape) != (B, E, H) or P.dtype != p_dtype or P.device != q.device):
         raise RuntimeError("attn must be the [batch, edges, heads] tensor the forward returned")
 
 

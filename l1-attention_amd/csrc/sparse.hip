@@ -358,12 +358,13 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_fwd_src(
 // dst pass.  For every edge of the dst:  dp = v[src].dvo[dst] (+ vb[dst].dvo[src] for bidi);
 // S = sum p*dp;  dq[dst] = scale * sum sign(q-k) * p * (dp - S)  accumulated as X - S*Y in one walk;
 // bidi: dvb[dst] = sum p * dvo[src].  Leaves da = p*(dp - S) (or p*dp) per edge in DA.
-template <typename T, int VEC, int MC, bool BIDI, int NWV>
+// ST: type of the rows in memory (S is the softmax sum below)
+template <typename T, int VEC, int MC, bool BIDI, int NWV, typename ST>
 __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_dst(
-    const T* __restrict__ dvo, const T* __restrict__ v, const T* __restrict__ vbk, const T* __restrict__ q,
-    const T* __restrict__ k, const int* __restrict__ dst_ptr, const int* __restrict__ csr_src,
+    const ST* __restrict__ dvo, const ST* __restrict__ v, const ST* __restrict__ vbk, const ST* __restrict__ q,
+    const ST* __restrict__ k, const int* __restrict__ dst_ptr, const int* __restrict__ csr_src,
     const int* __restrict__ long_list, const int* __restrict__ n_long, const T* __restrict__ P,
-    T* __restrict__ DA, T* __restrict__ dq, T* __restrict__ dvb, Geo g, int use_softmax, T scale)
+    T* __restrict__ DA, ST* __restrict__ dq, ST* __restrict__ dvb, Geo g, int use_softmax, T scale)
 {
 	extern __shared__ unsigned char smem_raw[];
 	T* smem = reinterpret_cast<T*>(smem_raw);
@@ -372,10 +373,10 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_dst(
 	if (!wave_item<NWV>(g, dst_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowq = (int64_t)g.H * g.W, rowv = (int64_t)g.H * g.Wv;
-	const T* qb = q + (int64_t)b * g.Tn * rowq;
-	const T* kb = k + (int64_t)b * g.Tn * rowq;
-	const T* vb_ = v + (int64_t)b * g.Tn * rowv;
-	const T* dvob = dvo + (int64_t)b * g.Tn * rowv;
+	const ST* qb = q + (int64_t)b * g.Tn * rowq;
+	const ST* kb = k + (int64_t)b * g.Tn * rowq;
+	const ST* vb_ = v + (int64_t)b * g.Tn * rowv;
+	const ST* dvob = dvo + (int64_t)b * g.Tn * rowv;
 	const T* Pb = P + (int64_t)b * g.E * g.H;
 	T* DAb = DA + (int64_t)b * g.E * g.H;
 
@@ -477,12 +478,12 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_dst(
 }
 
 // src pass: dv[src] = sum p * dvo[dst];  dk[src] = -scale * sum sign(q[dst]-k[src]) * da
-template <typename T, int VEC, int MC, int NWV>
+template <typename T, int VEC, int MC, int NWV, typename S>
 __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_src(
-    const T* __restrict__ dvo, const T* __restrict__ q, const T* __restrict__ k, const int* __restrict__ src_ptr,
+    const S* __restrict__ dvo, const S* __restrict__ q, const S* __restrict__ k, const int* __restrict__ src_ptr,
     const int* __restrict__ csc_dst, const int* __restrict__ csc_slot, const int* __restrict__ long_list,
-    const int* __restrict__ n_long, const T* __restrict__ P, const T* __restrict__ DA, T* __restrict__ dv,
-    T* __restrict__ dk, Geo g, T scale)
+    const int* __restrict__ n_long, const T* __restrict__ P, const T* __restrict__ DA, S* __restrict__ dv,
+    S* __restrict__ dk, Geo g, T scale)
 {
 	extern __shared__ unsigned char smem_raw[];
 	T* smem = reinterpret_cast<T*>(smem_raw);
@@ -491,8 +492,8 @@ __global__ __launch_bounds__(NWV == 1 ? 256 : 64 * NWV) void sparse_bwd_src(
 	if (!wave_item<NWV>(g, src_ptr, long_list, n_long, L)) return;
 	const int b = blockIdx.y, G = 1 << g.log2G;
 	const int64_t rowq = (int64_t)g.H * g.W, rowv = (int64_t)g.H * g.Wv;
-	const T* qb = q + (int64_t)b * g.Tn * rowq;
-	const T* dvob = dvo + (int64_t)b * g.Tn * rowv;
+	const S* qb = q + (int64_t)b * g.Tn * rowq;
+	const S* dvob = dvo + (int64_t)b * g.Tn * rowv;
 	const T* Pb = P + (int64_t)b * g.E * g.H;
 	const T* DAb = DA + (int64_t)b * g.E * g.H;
 	T kv[MC][VEC], dva[MC][VEC], dka[MC][VEC];
@@ -664,9 +665,9 @@ int sparse_fwd_impl(const S* v, const S* vbk, const S* q, const S* k, const void
 	return L1ATTN_OK;
 }
 
-template <typename T>
-int sparse_bwd_impl(const T* dvo, const T* v, const T* vbk, const T* q, const T* k, const void* plan, const T* P,
-                    T* dv, T* dvb, T* dq, T* dk, T* DA, Shape s, int use_softmax, bool bidi, hipStream_t st)
+template <typename T, typename S>
+int sparse_bwd_impl(const S* dvo, const S* v, const S* vbk, const S* q, const S* k, const void* plan, const T* P,
+                    S* dv, S* dvb, S* dq, S* dk, T* DA, Shape s, int use_softmax, bool bidi, hipStream_t st)
 {
 	if (s.B * s.T * s.H == 0) return L1ATTN_OK;
 	if (!dvo || !v || !q || !k || !plan || !dv || !dq || !dk || (s.E > 0 && (!P || !DA)) || (bidi && (!vbk || !dvb)))
@@ -678,20 +679,20 @@ int sparse_bwd_impl(const T* dvo, const T* v, const T* vbk, const T* q, const T*
 	const T scale = (T)(-1.0 / sqrt((double)s.W));
 	if (bidi) {
 #define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
-	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, true, N>), GRID, BLOCK, LDS, st, dvo, v, vbk, q, k, c.dst_ptr,   \
+	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, true, N, S>), GRID, BLOCK, LDS, st, dvo, v, vbk, q, k, c.dst_ptr,   \
 	                   c.csr_src, c.long_dst, c.n_long_dst, P, DA, dq, dvb, c.g, use_softmax, scale)
 		DISPATCH_VM(c, T, CALL);
 #undef CALL
 	} else {
 #define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
-	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, false, N>), GRID, BLOCK, LDS, st, dvo, v, vbk, q, k, c.dst_ptr,  \
+	hipLaunchKernelGGL((sparse_bwd_dst<T, V, M, false, N, S>), GRID, BLOCK, LDS, st, dvo, v, vbk, q, k, c.dst_ptr,  \
 	                   c.csr_src, c.long_dst, c.n_long_dst, P, DA, dq, dvb, c.g, use_softmax, scale)
 		DISPATCH_VM(c, T, CALL);
 #undef CALL
 	}
 	L1_LAUNCH_CHECK();
 #define CALL(V, M, N, GRID, BLOCK, LDS)                                                                         \
-	hipLaunchKernelGGL((sparse_bwd_src<T, V, M, N>), GRID, BLOCK, LDS, st, dvo, q, k, c.src_ptr, c.csc_dst,      \
+	hipLaunchKernelGGL((sparse_bwd_src<T, V, M, N, S>), GRID, BLOCK, LDS, st, dvo, q, k, c.src_ptr, c.csc_dst,      \
 	                   c.csc_slot, c.long_src, c.n_long_src, P, (const T*)DA, dv, dk, c.g, scale)
 	DISPATCH_VM(c, T, CALL);
 #undef CALL
@@ -715,7 +716,7 @@ extern "C" {
 	                            const TYPE* P, TYPE* dv, TYPE* dq, TYPE* dk, TYPE* DA, int64_t B, int64_t T,        \
 	                            int64_t H, int64_t W, int64_t Wv, int64_t E, int use_softmax, void* stream)         \
 	{                                                                                                               \
-		return sparse_bwd_impl<TYPE>(dvo, v, nullptr, q, k, plan, P, dv, nullptr, dq, dk, DA,                       \
+		return sparse_bwd_impl<TYPE, TYPE>(dvo, v, nullptr, q, k, plan, P, dv, nullptr, dq, dk, DA,                       \
 		                             Shape{B, T, H, W, Wv, E}, use_softmax, false, (hipStream_t)stream);            \
 	}                                                                                                               \
 	int l1attn_sparse_bidi_fwd_##SFX(const TYPE* vf, const TYPE* vb, const TYPE* q, const TYPE* k,                  \
@@ -730,14 +731,14 @@ extern "C" {
 	                                 TYPE* dq, TYPE* dk, TYPE* DA, int64_t B, int64_t T, int64_t H, int64_t W,      \
 	                                 int64_t Wv, int64_t E, int use_softmax, void* stream)                          \
 	{                                                                                                               \
-		return sparse_bwd_impl<TYPE>(dvo, vf, vb, q, k, plan, P, dvf, dvb, dq, dk, DA, Shape{B, T, H, W, Wv, E},    \
+		return sparse_bwd_impl<TYPE, TYPE>(dvo, vf, vb, q, k, plan, P, dvf, dvb, dq, dk, DA, Shape{B, T, H, W, Wv, E},    \
 		                             use_softmax, true, (hipStream_t)stream);                                       \
 	}
 
 L1_SPARSE_ENTRY(f32, float)
 L1_SPARSE_ENTRY(f64, double)
 
-// Forward only with 16-bit rows (the reference dispatches its forward kernels for Half as well,
+// Forward with 16-bit rows (the reference dispatches its forward kernels for Half as well,
 // cuda/l1attn_sparse_cuda_kernel.cu:405-435 and :684-714, and its backward kernels for float and double
 // only, :483-519): v, q, k and vo are IEEE half (f16) or bfloat16 (bf16) in memory, the logits, the
 // softmax and the value sums run in fp32, the weights P are fp32.
@@ -761,5 +762,31 @@ L1_SPARSE_ENTRY(f64, double)
 
 L1_SPARSE_FWD16_ENTRY(f16, f16_t)
 L1_SPARSE_FWD16_ENTRY(bf16, bf16_t)
+
+// Backward with 16-bit rows (an addition: the reference's backward launchers take float and double only):
+// dvo, v/vf, vb, q, k and the gradients dv/dvf, dvb, dq, dk are 16-bit in memory, P and DA fp32, every sum fp32,
+// each gradient element rounded once on store.
+#define L1_SPARSE_BWD16_ENTRY(SFX, STYPE)                                                                           \
+	int l1attn_sparse_bwd_##SFX(const void* dvo, const void* v, const void* q, const void* k, const void* plan,     \
+	                            const float* P, void* dv, void* dq, void* dk, float* DA, int64_t B, int64_t T,      \
+	                            int64_t H, int64_t W, int64_t Wv, int64_t E, int use_softmax, void* stream)         \
+	{                                                                                                               \
+		return sparse_bwd_impl<float, STYPE>((const STYPE*)dvo, (const STYPE*)v, nullptr, (const STYPE*)q,          \
+		                                     (const STYPE*)k, plan, P, (STYPE*)dv, nullptr, (STYPE*)dq, (STYPE*)dk, \
+		                                     DA, Shape{B, T, H, W, Wv, E}, use_softmax, false, (hipStream_t)stream); \
+	}                                                                                                               \
+	int l1attn_sparse_bidi_bwd_##SFX(const void* dvo, const void* vf, const void* vb, const void* q, const void* k, \
+	                                 const void* plan, const float* P, void* dvf, void* dvb, void* dq, void* dk,    \
+	                                 float* DA, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,  \
+	                                 int use_softmax, void* stream)                                                 \
+	{                                                                                                               \
+		return sparse_bwd_impl<float, STYPE>((const STYPE*)dvo, (const STYPE*)vf, (const STYPE*)vb,                 \
+		                                     (const STYPE*)q, (const STYPE*)k, plan, P, (STYPE*)dvf, (STYPE*)dvb,   \
+		                                     (STYPE*)dq, (STYPE*)dk, DA, Shape{B, T, H, W, Wv, E}, use_softmax,     \
+		                                     true, (hipStream_t)stream);                                            \
+	}
+
+L1_SPARSE_BWD16_ENTRY(f16, f16_t)
+L1_SPARSE_BWD16_ENTRY(bf16, bf16_t)
 
 }  // extern "C"

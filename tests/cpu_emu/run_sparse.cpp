@@ -26,21 +26,19 @@ static S* to_storage(const std::vector<float>& x)
 	return p;
 }
 
-template <typename S>
-static int backward(const int64_t*, const void*, const S*, const S*, const S*, const S*, const S*, const S*, FILE*)
-{
-	return 0;  // the 16-bit types have no backward
-}
-#define L1_EMU_BWD(SFX, TYPE)                                                                                       \
-	template <>                                                                                                     \
-	int backward<TYPE>(const int64_t* d, const void* plan, const TYPE* dvo, const TYPE* vf, const TYPE* vb,         \
-	                   const TYPE* q, const TYPE* k, const TYPE* P, FILE* fo)                                       \
+// the backward of the storage type S (weights and scratch of type PT) on dvo and the weights just written
+#define L1_EMU_BWD(SFX, S, PT)                                                                                      \
+	static int backward(const int64_t* d, const void* plan, const S* dvo, const S* vf, const S* vb, const S* q,     \
+	                    const S* k, const PT* P, FILE* fo)                                                          \
 	{                                                                                                               \
 		const int64_t B = d[0], T = d[1], H = d[2], W = d[3], Wv = d[4], E = d[5];                                  \
 		const size_t nv = (size_t)(B * T * H * Wv), nq = (size_t)(B * T * H * W), ne = (size_t)(B * E * H);         \
-		auto al = [](size_t n) { return (TYPE*)aligned_alloc(16, (n * sizeof(TYPE) + 15) / 16 * 16 + 16); };        \
-		TYPE *dvf = al(nv), *dvb = al(nv), *dq = al(nq), *dk = al(nq), *DA = al(ne);                                \
-		for (size_t i = 0; i < nv; i++) dvb[i] = 0;                                                                 \
+		S* dvf = (S*)aligned_alloc(16, (nv * sizeof(S) + 15) / 16 * 16 + 16);                                       \
+		S* dvb = (S*)aligned_alloc(16, (nv * sizeof(S) + 15) / 16 * 16 + 16);                                       \
+		S* dq = (S*)aligned_alloc(16, (nq * sizeof(S) + 15) / 16 * 16 + 16);                                        \
+		S* dk = (S*)aligned_alloc(16, (nq * sizeof(S) + 15) / 16 * 16 + 16);                                        \
+		PT* DA = (PT*)aligned_alloc(16, (ne * sizeof(PT) + 15) / 16 * 16 + 16);                                     \
+		for (size_t i = 0; i < nv; i++) dvb[i] = (S)0.0f;                                                           \
 		const int rc = d[7] ? l1attn_sparse_bidi_bwd_##SFX(dvo, vf, vb, q, k, plan, P, dvf, dvb, dq, dk, DA, B, T,  \
 		                                                   H, W, Wv, E, (int)d[6], nullptr)                         \
 		                    : l1attn_sparse_bwd_##SFX(dvo, vf, q, k, plan, P, dvf, dq, dk, DA, B, T, H, W, Wv, E,    \
@@ -53,8 +51,10 @@ static int backward(const int64_t*, const void*, const S*, const S*, const S*, c
 		free(dvf); free(dvb); free(dq); free(dk); free(DA);                                                         \
 		return 0;                                                                                                   \
 	}
-L1_EMU_BWD(f32, float)
-L1_EMU_BWD(f64, double)
+L1_EMU_BWD(f32, float, float)
+L1_EMU_BWD(f64, double, double)
+L1_EMU_BWD(f16, f16_t, float)
+L1_EMU_BWD(bf16, bf16_t, float)
 
 template <typename S, typename P, typename F>
 static int run(const int64_t* d, const void* plan, const std::vector<float>& vf, const std::vector<float>& vb,
@@ -69,9 +69,9 @@ static int run(const int64_t* d, const void* plan, const std::vector<float>& vf,
 	if (rc) return 10 + (rc < 0 ? -rc : rc);
 	for (int64_t i = 0; i < B * T * H * Wv; i++) { const double x = (double)vo[i]; fwrite(&x, 8, 1, fo); }
 	for (int64_t i = 0; i < B * E * H; i++) { const double x = (double)pw[i]; fwrite(&x, 8, 1, fo); }
-	if (sizeof(S) == sizeof(P)) {  // float32 / float64: the backward on the weights just written
+	{
 		S* pdvo = to_storage<S>(dvo);
-		const int rcb = backward<S>(d, plan, pdvo, pvf, pvb, pq, pk, (const S*)pw, fo);
+		const int rcb = backward(d, plan, pdvo, pvf, pvb, pq, pk, (const P*)pw, fo);
 		free(pdvo);
 		if (rcb) return rcb;
 	}

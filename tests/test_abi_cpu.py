@@ -339,7 +339,7 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
         drv.sparse_forward(torch.zeros(B, T + 1, H, Wv), q, k, coo, 3, True)
     with pytest.raises(RuntimeError, match="only float32 and float64"):
         drv.dense_forward(q.half(), k.half())
-    # 16-bit rows: forward only, fp32 edge weights, the entry point named after the storage type
+    # 16-bit rows: fp32 edge weights, entry points named after the storage type
     for dt, sfx in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
         v16, vb16, q16, k16 = (x.to(dt) for x in (v, vb, q, k))
         del _FakeLib.calls[:]
@@ -349,10 +349,12 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
         vo, P = drv.bidi_forward(v16, vb16, q16, k16, coo, 3, False)
         assert _FakeLib.calls[-1] == "l1attn_sparse_bidi_fwd_" + sfx
         assert vo.dtype == dt and P.dtype == torch.float32
-        with pytest.raises(RuntimeError, match="backward is not implemented"):
-            drv.sparse_backward(torch.zeros_like(v16), v16, q16, k16, coo, P, 3, True)
-        with pytest.raises(RuntimeError, match="backward is not implemented"):
-            drv.bidi_backward(torch.zeros_like(v16), v16, vb16, q16, k16, coo, P, 3, True)
+        grads = drv.sparse_backward(torch.zeros_like(v16), v16, q16, k16, coo, P, 3, True)
+        assert _FakeLib.calls[-1] == "l1attn_sparse_bwd_" + sfx and all(g_.dtype == dt for g_ in grads)
+        grads = drv.bidi_backward(torch.zeros_like(v16), v16, vb16, q16, k16, coo, P, 3, True)
+        assert _FakeLib.calls[-1] == "l1attn_sparse_bidi_bwd_" + sfx and len(grads) == 4
+        with pytest.raises(RuntimeError, match="attn must be"):  # the weights of a 16-bit call are fp32
+            drv.sparse_backward(torch.zeros_like(v16), v16, q16, k16, coo, P.to(dt), 3, True)
         with pytest.raises(RuntimeError, match="share dtype"):
             drv.sparse_forward(v, q16, k16, coo, 3, True)
 

@@ -1,7 +1,7 @@
 """CPU run of the sparse and bidirectional kernels, forward and backward (csrc/sparse.hip compiled for the host against
 tests/cpu_emu/hip/hip_runtime.h: GPU threads are OS threads, cross-lane reads, fences and __syncthreads() are
-barriers) under AddressSanitizer, for float32, float64 and (forward) float16 and bfloat16 rows, against fp64
-closed forms and torch autograd through them.
+barriers) under AddressSanitizer, for float32, float64, float16 and bfloat16 rows, against fp64 closed forms
+and torch autograd through them.
 
 It covers what the 16-bit entry points add to kernels that the GPU tests already cover in float32 and float64:
 conversion on load, rounding on store, 8-byte row pieces, and the claim their GPU test rests on -- that the
@@ -81,8 +81,7 @@ def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind):
     vo = torch.from_numpy(raw[:nv].copy()).view(B, T, H, Wv)
     P = torch.from_numpy(raw[nv:nv + B * E * H].copy()).view(B, E, H)
     slot_row = torch.from_numpy(arrays[3].astype(np.int64))  # original row of each slot
-    _run.grads = None
-    if kind in ("f32", "f64"):  # the driver also ran the backward on dvo
+    if True:  # the driver also ran the backward on dvo (rounded to the storage type)
         pos, nq = nv + B * E * H, B * T * H * W
         take = lambda n, shape: torch.from_numpy(raw[pos:pos + n].copy()).view(*shape)
         dvf = take(nv, (B, T, H, Wv)); pos += nv
@@ -90,7 +89,8 @@ def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind):
         dq = take(nq, (B, T, H, W)); pos += nq
         dk = take(nq, (B, T, H, W)); pos += nq
         assert pos == raw.shape[0]
-        _run.grads = (dvo.double(), dvf, dvb, dq, dk)
+        dvo_s = dvo.to(TORCH_T[kind]) if kind in TORCH_T else dvo
+        _run.grads = (dvo_s.double(), dvf, dvb, dq, dk)
     return vo, P, slot_row
 
 
@@ -131,10 +131,12 @@ def test_sparse_forward_kernels_on_cpu(runner, tmp_path, shape, sm):
         vo16, P16, _ = _run(runner, tmp_path, vf, vb, q, k, co, sm, False, kind)
         assert torch.equal(P16, P32)
         assert torch.equal(vo16.float(), vo32.float().to(dt).float())
+        _check_grads(vf, vb, q, k, co, sm, False, TOL[kind])  # 16-bit gradients: one rounding on store
         # bidirectional: tolerance of the 16-bit type against the closed form
         vob, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, sm, True, kind)
         ref = cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, sm)
         assert cf.rel_err(vob, ref) <= TOL[kind]
+        _check_grads(vf, vb, q, k, co, sm, True, TOL[kind])
     # float64, both operators, forward and backward
     for bidi in (False, True):
         vo, _, _ = _run(runner, tmp_path, vf, vb, q, k, co, sm, bidi, "f64")

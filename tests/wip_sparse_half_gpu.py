@@ -1,5 +1,6 @@
-"""GPU parity of the sparse and bidirectional forwards with 16-bit rows (float16, bfloat16), through
-the reference's Python API and so through l1attn_sparse_fwd_{f16,bf16} / l1attn_sparse_bidi_fwd_*.
+"""GPU parity of the sparse and bidirectional operators with 16-bit rows (float16, bfloat16), forward and
+backward, through the reference's Python API and so through l1attn_sparse_{fwd,bwd}_{f16,bf16} /
+l1attn_sparse_bidi_{fwd,bwd}_*.
 
 This file has not run on a GPU yet, which is why its name keeps it out of pytest's collection
 (run it as `python -m pytest tests/wip_sparse_half_gpu.py -m gpu`); rename it to test_*.py once
@@ -151,19 +152,47 @@ def test_half_forward_benchmark_geometry(dt, which):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-def test_half_backward_raises_and_empty_list(dt):
-    print("case sparse 16-bit backward / empty list", dt, flush=True)
+@pytest.mark.parametrize("shape", [(2, 9, 3, 5, 5, 40), (1, 64, 8, 32, 32, 900), (2, 50, 4, 64, 64, 700),
+                                   (2, 20, 3, 8, 12, 90)])
+@pytest.mark.parametrize("sm", [True, False])
+def test_half_backward_vs_autograd_closed_form(dt, shape, sm):
+    """Gradients of both operators with 16-bit rows (sums in fp32, one rounding per gradient element) against
+    torch autograd through the fp64 closed form on the same 16-bit-valued inputs: 2^-10 / 2^-7 of the largest
+    gradient; bitwise run-to-run."""
+    B, T, H, W, Wv, E = shape
+    print("case sparse 16-bit backward", dt, shape, sm, flush=True)
+    sp, bi = _m()
+    g = torch.Generator().manual_seed(sum(shape) + 3)
+    co = torch.randint(0, T, (E, 2), generator=g)
+    coo, dmx, _ = oracle.expand_coo(co)
+    cood = coo.cuda()
+    q, k, (vf, vb, dvo) = _inputs(B, T, H, W, Wv, dt, g, n_v=3)
+    x = [t.double().requires_grad_() for t in (vf, vb, q, k)]
+    ref_u = torch.autograd.grad(cf.sparse_value(x[0], x[2], x[3], coo, sm), (x[0], x[2], x[3]), dvo.double())
+    ref_b = torch.autograd.grad(cf.bidi_value(x[0], x[1], x[2], x[3], coo, sm), x, dvo.double())
+    c = lambda t: t.cuda().to(dt).requires_grad_()
+    a, qd, kd = c(vf), c(q), c(k)
+    got = torch.autograd.grad(sp.L1AttnSparseFn.apply(a, qd, kd, cood, dmx, sm), (a, qd, kd), dvo.cuda().to(dt))
+    for u, r in zip(got, ref_u):
+        assert u.dtype == dt and cf.rel_err(u.float().cpu(), r) <= TOL[dt]
+    a, b, qd, kd = c(vf), c(vb), c(q), c(k)
+    got = torch.autograd.grad(bi.L1AttnSparseBidiFn.apply(a, b, qd, kd, cood, dmx, sm), (a, b, qd, kd),
+                              dvo.cuda().to(dt))
+    for u, r in zip(got, ref_b):
+        assert cf.rel_err(u.float().cpu(), r) <= TOL[dt]
+    again = torch.autograd.grad(bi.L1AttnSparseBidiFn.apply(a, b, qd, kd, cood, dmx, sm), (a, b, qd, kd),
+                                dvo.cuda().to(dt))
+    assert all(torch.equal(u, w) for u, w in zip(got, again))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_half_empty_list(dt):
+    print("case sparse 16-bit empty list", dt, flush=True)
     sp, bi = _m()
     x = torch.randn(1, 4, 2, 8).cuda().to(dt)
-    coo = torch.tensor([[0, 1, 0, 0], [2, 0, 0, 0]], dtype=torch.int32).cuda()
-    xr = x.clone().requires_grad_()
-    vo = sp.L1AttnSparse()(xr, xr, xr, coo, 1)
-    with pytest.raises(RuntimeError, match="backward is not implemented"):
-        vo.float().sum().backward()
-    xr = x.clone().requires_grad_()
-    vo = bi.L1AttnSparseBidi()(xr, xr, xr, xr, coo, 1)
-    with pytest.raises(RuntimeError, match="backward is not implemented"):
-        vo.float().sum().backward()
     coo0 = torch.zeros(0, 4, dtype=torch.int32).cuda()
-    vo = sp.L1AttnSparse()(x, x, x, coo0, 1)
+    xr = x.clone().requires_grad_()
+    vo = sp.L1AttnSparse()(xr, xr, xr, coo0, 1)
     assert vo.dtype == dt and torch.count_nonzero(vo) == 0
+    vo.float().sum().backward()
+    assert torch.count_nonzero(xr.grad) == 0
