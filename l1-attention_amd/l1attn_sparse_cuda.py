@@ -7,6 +7,8 @@
 
 The reference's README calls the module with five arguments (README.md:93) while its wrapper
 requires six (cuda/l1attn_sparse_cuda.py:54); both forms are accepted here.
+float32 and float64 as in the reference; float16 and bfloat16 tensors are accepted too (rows and
+gradients in that type, sums and edge weights in fp32; the reference dispatches Half in its forward only).
 """
 import torch
 from torch import nn
