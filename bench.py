@@ -1,7 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the L1-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-sparse] [--skip-cpu] [--extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-sparse] [--skip-cpu]
+    python bench.py --sweep                     # the reference's own timing grid (benchmark.py:57-66), one JSON line per cell
+    python bench.py --skip-dense --only config4 # one sparse configuration per process (profiling aid)
+    python bench.py --extra                     # opt-in legs: fused operator, 16-bit rows, fixed-point forward
 
 A step is one dense L1Attn forward + backward (through the reference's Python API,
 l1attn_cuda.L1AttnFn) over the headline configuration  q,k fp32 [B=8, T=4096, H=16, W=64],
@@ -34,6 +37,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # KiB per kernel, fetch / write: column ranks 149986 / 262144, main kernel 10683411 / 8652097,
 # column-sum reduce 65547 / 2048, dk reduce 1050658 / 131072.
 DENSE_BWD_TRAFFIC_BYTES = ((149986 + 10683411 + 65547 + 1050658) * 2 + 262144 + 8652097 + 2048 + 131072) * 1024
+# The figure above is NOT measured by the run that prints it: it is read off committed counter summaries.
+DENSE_BWD_TRAFFIC_SOURCE = {
+    "measured_in_this_run": False,
+    "files": ["profiles/dense_B8_T4096_H16_W64_pmc_fetch_size.txt", "profiles/dense_B8_T4096_H16_W64_pmc_write_size.txt",
+              "profiles/copy_1GiB_pmc_fetch_size.txt", "profiles/copy_1GiB_pmc_write_size.txt"],
+    "collected_at_commit": "65a21ba",
+    "kernel_state": "one change before the current backward kernel: the later dst tiles of a workgroup then loaded, "
+                    "added and stored their dk partial rows; they now send adds to the L2 instead",
+}
 
 
 def log(*a):
@@ -105,9 +117,11 @@ def time_gpu(fn, iters, warm=2):
     return e0.elapsed_time(e1) / iters
 
 
-def sparse_configs(skip_cpu):
+def sparse_configs(skip_cpu, only=None):
     """Configuration 4 (one-directional, B4 T4096 H8 W32, degree U{1..64}) and configuration 5
-    (bidirectional, B1 T65536 H4 W64, Zipf degrees + self loops): fwd+bwd through the Python API."""
+    (bidirectional, B1 T65536 H4 W64, Zipf degrees + self loops): fwd+bwd through the Python API.
+    `only`: "config4" or "config5" runs that one alone, so that a profile of the process holds one configuration's
+    launches and its kernel times and HBM counters can be read per configuration."""
     import torch
     import workloads
     import l1attn_sparse_cuda as sp
@@ -116,8 +130,11 @@ def sparse_configs(skip_cpu):
     dev = torch.device("cuda:0")
     res = {}
     for name, bidi, (B, T, H, W), co in (
-            ("config4_uni", False, (4, 4096, 8, 32), workloads.uniform_degree_graph(4096, 64, seed=1004)),
-            ("config5_bidi", True, (1, 65536, 4, 64), workloads.powerlaw_graph(65536, seed=1005))):
+            ("config4_uni", False, (4, 4096, 8, 32), lambda: workloads.uniform_degree_graph(4096, 64, seed=1004)),
+            ("config5_bidi", True, (1, 65536, 4, 64), lambda: workloads.powerlaw_graph(65536, seed=1005))):
+        if only and not name.startswith(only):
+            continue
+        co = co() if callable(co) else co
         E = co.shape[0]
         cod = co.to(dev)
         ms_expand = time_gpu(lambda: sp.expandCoo(cod, warn=False), 3, warm=1)
@@ -160,6 +177,12 @@ def sparse_configs(skip_cpu):
             "bytes_alg": bytes_alg, "alg_GBps": bytes_alg / (ms * 1e-3) / 1e9,
             "frac_of_hbm_peak": bytes_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "bytes_min": bytes_min, "min_GBps": bytes_min / (ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak_bytes_min": bytes_min / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "working_set_bytes": 11 * T * r,
+            "where_the_rows_live": "the eleven [B,T,H,W] tensors of a fwd+bwd are %.0f MiB: they stay in the L2s / the "
+                                   "256 MiB Infinity Cache between gathers, so alg_GBps is a cache-bandwidth figure "
+                                   "of the gather model, not HBM traffic; HBM sees about bytes_min per fwd+bwd"
+                                   % (11 * T * r / 2.0 ** 20),
             "expand_coo_gpu_ms": ms_expand, "expand_coo_cpu_oracle_ms": cpu_expand_ms,
             "note": "plan build (two radix sorts) is cached per edge list and excluded from fwd/bwd time",
         }
@@ -178,6 +201,8 @@ def extra_legs():
     import l1attn_cuda
     import l1attn_sparse_cuda as sp
     import l1attn_sparse_bidi_cuda as bi
+    import _l1attn_hip as drv
+    drv.enable_experimental("fused", "rows16", "fixed")  # these legs exist to time exactly those paths
     dev = torch.device("cuda:0")
     res = {"fused_forward": {}, "sparse_16bit": {}}
     for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
@@ -252,7 +277,6 @@ def extra_legs():
             row[name_dt + "_fwd_bwd_ms"] = time_gpu(fwdbwd, 10)
         res["sparse_16bit"][name] = row
         log(name, json.dumps(row))
-    import _l1attn_hip as drv
     res["fixed_point_forward"] = {}
     for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
         q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
@@ -298,6 +322,48 @@ def instruction_rates():
         rates[name] = {"ms": ms, "steps_per_simd_ns": steps / (256 * 4) / (ms * 1e6),
                        "lane_steps_tops": steps * 64 / (ms * 1e-3) / 1e12}
     return rates
+
+
+def reference_sweep(num_runs=10):
+    """The reference's own timing grid (benchmark.py:57-66): B=512, H=8, T in {16,...,256}, W in
+    {16,32,33,64,65,96,97,128}, forward and backward of L1AttnFn timed separately as averages over num_runs.
+    Differences from that script, on purpose: HIP events on the stream instead of perf_counter around
+    synchronize (its numbers at these sizes are mostly launch and sync latency), inputs made once per cell,
+    and each cell also reports algorithmic Tops/s.  One JSON line per cell on stdout, and the list as return value."""
+    import torch
+    import l1attn_cuda
+    dev = torch.device("cuda:0")
+    B, H = 512, 8
+    rows = []
+    for T in (16, 32, 64, 128, 256):
+        for W in (16, 32, 33, 64, 65, 96, 97, 128):
+            g = torch.Generator(device=dev).manual_seed(1000 + T * 1000 + W)
+            q = torch.randn(B, T, H, W, device=dev, generator=g).requires_grad_()
+            k = torch.randn(B, T, H, W, device=dev, generator=g).requires_grad_()
+            dA = torch.randn(B, T, T, H, device=dev, generator=g)
+            attn = l1attn_cuda.L1AttnFn.apply(q, k)
+            attn.backward(dA)  # warm-up of both launches (workspace allocation, plan choice)
+            torch.cuda.synchronize()
+            ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(num_runs)]
+            for e in ev:
+                q.grad = None
+                k.grad = None
+                e[0].record()
+                attn = l1attn_cuda.L1AttnFn.apply(q, k)
+                e[1].record()
+                attn.backward(dA)
+                e[2].record()
+            torch.cuda.synchronize()
+            fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / num_runs
+            bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / num_runs
+            N = B * T * T * H * W
+            row = {"sweep": "benchmark.py:57-66", "batch_size": B, "seq_length": T, "n_heads": H, "width": W,
+                   "avg_forward_ms": fwd_ms, "avg_backward_ms": bwd_ms,
+                   "fwd_tops": 2 * N / fwd_ms / 1e9, "bwd_tops": 4 * N / bwd_ms / 1e9}
+            print(json.dumps(row), flush=True)
+            rows.append(row)
+            del q, k, dA, attn
+    return rows
 
 
 def valu_probe():
@@ -379,6 +445,10 @@ def main():
     ap.add_argument("--skip-sparse", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-dense", action="store_true", help="profiling aid: sparse legs only")
+    ap.add_argument("--only", choices=("config4", "config5"), default=None,
+                    help="with the sparse legs: run this configuration alone (one per process for profiles)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="only run the reference's timing grid (benchmark.py:57-66), one JSON line per cell")
     ap.add_argument("--extra", action="store_true",
                     help="only time the fused forward and the 16-bit sparse forwards beside what they replace")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -406,7 +476,10 @@ def main():
         print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "copies": 3}))
         return
     if args.skip_dense:
-        print(json.dumps({"sparse": sparse_configs(True)}), flush=True)
+        print(json.dumps({"sparse": sparse_configs(True, args.only)}), flush=True)
+        return
+    if args.sweep:
+        reference_sweep()
         return
     if args.extra:
         print(json.dumps({"extra": extra_legs()}), flush=True)
@@ -420,7 +493,8 @@ def main():
         "bound": "valu", "kernel": "dense_bwd_f32_fast (+ dense_column_ranks, dense_bwd_reduce_colsum, dense_bwd_reduce_dk: one backward launch)",
         "achieved": d["bwd_tops"], "peak": P_VALU_TOPS, "unit": "TFLOP/s",
         "frac": d["bwd_tops"] / P_VALU_TOPS,
-        "traffic": DENSE_BWD_TRAFFIC_BYTES,
+        "traffic": DENSE_BWD_TRAFFIC_BYTES, "traffic_source": DENSE_BWD_TRAFFIC_SOURCE,
+        "frac_of_datasheet_fp32": d["bwd_tops"] / 157.3,
         "flops_per_launch": 4 * N, "avg_launch_ms": d["bwd_ms"],
         "note": "algorithmic ops (4 per pair-element) over the HIP-event time of the backward launch; "
                 "peak = nominal fp32 VALU issue rate (one wave64 instruction per SIMD every 2 cycles at "
@@ -444,7 +518,7 @@ def main():
     }
     if not args.skip_sparse:
         log("sparse configurations ...")
-        out["sparse"] = sparse_configs(args.skip_cpu)
+        out["sparse"] = sparse_configs(args.skip_cpu, args.only)
     if not args.skip_cpu:
         log("cpu baseline ...")
         out["cpu_baseline"] = cpu_baseline()

@@ -34,21 +34,6 @@ extern "C" {
 /* Library version (major*10000 + minor*100 + patch). */
 int l1attn_version(void);
 
-/*
- * Measurement aid, no counterpart in the reference: a register-only loop of independent,
- * non-packed v_fmac_f32 (blocks workgroups of 512 threads, every wave issues iters*64 of them),
- * to time what the fp32 VALU of the GPU at hand sustains for ordinary code against the nominal
- * one instruction per SIMD every two cycles.  out: blocks*512 floats.  Asynchronous.
- */
-int l1attn_probe_valu(float* out, int64_t blocks, int64_t iters, void* stream);
-/*
- * The same probe for other instructions (same geometry and accounting), to learn an instruction's
- * issue rate before a kernel is built on it: op 0 = v_fmac_f32 (as above), 1 = v_sad_u32 (|a-b|+c on
- * unsigned integers in one instruction) on VGPRs, 2 = v_sad_u32 with an SGPR operand, 3 = pairs of
- * v_sub_f32 and v_add_f32 |x| (2 instructions per counted step).  No counterpart in the reference.
- */
-int l1attn_probe_valu_op(float* out, int64_t blocks, int64_t iters, int op, void* stream);
-
 /* ------------------------------------------------------------------------------ dense */
 
 /*
@@ -343,6 +328,27 @@ int l1attn_sparse_bidi_bwd_bf16(const void* dvo, const void* vf, const void* vb,
                                 void* dvf, void* dvb, void* dq, void* dk, float* DA,
                                 int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,
                                 int use_softmax, void* stream);
+
+/* ------------------------------------------- measurement aids (bench.py only) */
+/*
+ * Not part of the operator boundary and no counterpart in the reference: nothing in the operators calls
+ * these, a binding of the reference would not declare them.  They time instruction issue rates on the GPU at
+ * hand so that the bench line can state what its roofline denominator means on that box.
+ */
+/*
+ * A register-only loop of independent,
+ * non-packed v_fmac_f32 (blocks workgroups of 512 threads, every wave issues iters*64 of them),
+ * to time what the fp32 VALU of the GPU at hand sustains for ordinary code against the nominal
+ * one instruction per SIMD every two cycles.  out: blocks*512 floats.  Asynchronous.
+ */
+int l1attn_probe_valu(float* out, int64_t blocks, int64_t iters, void* stream);
+/*
+ * The same probe for other instructions (same geometry and accounting), to learn an instruction's
+ * issue rate before a kernel is built on it: op 0 = v_fmac_f32 (as above), 1 = v_sad_u32 (|a-b|+c on
+ * unsigned integers in one instruction) on VGPRs, 2 = v_sad_u32 with an SGPR operand, 3 = pairs of
+ * v_sub_f32 and v_add_f32 |x| (2 instructions per counted step).  No counterpart in the reference.
+ */
+int l1attn_probe_valu_op(float* out, int64_t blocks, int64_t iters, int op, void* stream);
 
 #ifdef __cplusplus
 }

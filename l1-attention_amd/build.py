@@ -28,26 +28,72 @@ def _sregs(tok):
     return {int(m.group(1))} if m else set()
 
 
-def check_scalar_prefetch(asm_text, kernel_substr="dense_fwd_f32_pipe"):
-    """Static check of the generated ISA of the software-pipelined forward kernels.
+_VMEM_LOAD = re.compile(r"^(buffer_load|global_load|flat_load|scratch_load|tbuffer_load|ds_read|ds_load|"
+                        r"buffer_atomic|global_atomic|flat_atomic|ds_\w+_rtn)")
 
-    Those kernels issue `s_load_dwordx16` from inline asm and wait for it one chunk of math later.
+
+def _walk_kernels(asm_text):
+    """(kernel, line number, instruction text, inside an inline-asm block) for every instruction of a device
+    listing.  The compiler brackets inline asm with `;;#ASMSTART` / `;;#ASMEND` comment lines."""
+    cur, in_asm = None, False
+    for ln, line in enumerate(asm_text.split("\n"), 1):
+        l = line.strip()
+        if l.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if l.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if l.startswith("_Z") and ":" in l.split(";")[0]:
+            cur, in_asm = l.split(":")[0], False
+            continue
+        if cur is None or not l or l[0] in ";.":
+            continue
+        l = l.split(";")[0].strip()
+        if l:
+            yield cur, ln, l, in_asm
+
+
+def check_inline_asm_loads(asm_text, where=""):
+    """No inline-asm block of any kernel may issue a load whose result arrives later (vector memory, LDS, or an
+    atomic that returns a value): the compiler does not know that the destination registers are still being
+    written, is free to move or reuse them before the hand-placed wait, and the late data then lands in whatever
+    lives there (an address, an exec mask) -- a memory fault on the GPU.  Loads of that kind go through builtins
+    or plain C++, which the compiler tracks.  The one exception, scalar loads, is checked instruction by
+    instruction in check_scalar_prefetch.  Returns the set of kernels whose inline asm issues scalar loads."""
+    problems, with_sload = [], set()
+    for kern, ln, l, in_asm in _walk_kernels(asm_text):
+        if not in_asm:
+            continue
+        op = l.split()[0]
+        if _VMEM_LOAD.match(op):
+            problems.append("%s line %d: %s" % (kern, ln, l))
+        elif op.startswith("s_load_") or op.startswith("s_buffer_load"):
+            with_sload.add(kern)
+    if problems:
+        raise RuntimeError("inline asm issues loads the compiler does not track (%s):\n%s"
+                           % (where or "device code", "\n".join(problems[:10])))
+    return with_sload
+
+
+def check_scalar_prefetch(asm_text, kernels=None):
+    """Static check of the scalar loads in the generated ISA, meant for the kernels that issue them from
+    inline asm and cheap enough to run on every kernel.
+
+    The pipelined forward kernels issue `s_load_dwordx16` from inline asm and wait for it one chunk of math later.
     The compiler does not know that the destination SGPRs are written asynchronously: if register
     pressure makes it spill, copy or reuse them between the load and the next `s_waitcnt lgkmcnt(0)`,
     the late-arriving data lands in whatever lives there by then (a pointer, an exec mask) and the
-    kernel faults.  This walks every such kernel and fails the build if any instruction reads or
+    kernel faults.  This walks the kernels (`kernels`: a set of mangled names, default: every kernel of the
+    listing; straight-line order, which is how both the compiler and the helper lay loads and waits out) and
+    fails the build if any instruction reads or
     writes an SGPR that still has a scalar load in flight, or if the kernel ends with one in flight.
-    Returns the number of prefetch loads checked."""
+    Returns the number of scalar loads checked."""
     cur, inflight, n_loads, problems = None, set(), 0, []
-    for ln, line in enumerate(asm_text.split("\n"), 1):
-        l = line.strip()
-        if l.startswith("_Z") and ":" in l.split(";")[0]:
-            cur, inflight = l.split(":")[0], set()
-            continue
-        if cur is None or kernel_substr not in cur or not l or l[0] in ";.":
-            continue
-        l = l.split(";")[0].strip()
-        if not l:
+    for kern, ln, l, _ in _walk_kernels(asm_text):
+        if kern != cur:
+            cur, inflight = kern, set()
+        if kernels is not None and cur not in kernels:
             continue
         op = l.split()[0]
         toks = re.findall(r"s\[\d+:\d+\]|s\d+", l)
@@ -74,6 +120,43 @@ def check_scalar_prefetch(asm_text, kernel_substr="dense_fwd_f32_pipe"):
         msg = "\n".join("%s line %d: %s" % p for p in problems[:10])
         raise RuntimeError("scalar-prefetch check failed: SGPRs touched while their s_load is in flight\n" + msg)
     return n_loads
+
+
+_ASM_STMT = re.compile(r"\basm\s*(?:volatile\s*)?\(")
+SCALAR_LOAD_HELPER = ("dense.hip", "sload32")  # the one function whose inline asm may issue scalar loads
+
+
+def check_asm_sources(files=None):
+    """Source-level twin of check_inline_asm_loads, so that the rule also covers templates nobody instantiates
+    yet: no `asm` statement under csrc/ may contain a vector-memory, LDS or returning-atomic load, and `s_load`
+    may appear only in the body of the one helper named above.  `files`: {name: text}, default csrc/*."""
+    if files is None:
+        files = {}
+        for path in sorted(glob.glob(os.path.join(HERE, "csrc", "*"))):
+            if path.endswith((".hip", ".h")):
+                with open(path) as f:
+                    files[os.path.basename(path)] = f.read()
+    problems = []
+    for name, text in sorted(files.items()):
+        for m in _ASM_STMT.finditer(text):
+            depth, i = 1, m.end()
+            while i < len(text) and depth:  # the statement up to its closing parenthesis
+                depth += {"(": 1, ")": -1}.get(text[i], 0)
+                i += 1
+            body = " ".join(re.findall(r'"((?:[^"\\]|\\.)*)"', text[m.end():i]))
+            line = text.count("\n", 0, m.start()) + 1
+            for ins in re.split(r"\\n|\\t|;", body):
+                op = ins.strip().split(" ")[0]
+                if _VMEM_LOAD.match(op):
+                    problems.append("%s:%d: inline asm issues %s" % (name, line, op))
+                elif op.startswith("s_load_") or op.startswith("s_buffer_load"):
+                    # the enclosing function: the last definition header before the statement
+                    heads = re.findall(r"\b(\w+)\s*\([^;{}]*\)\s*\{", text[:m.start()])
+                    if (name, heads[-1] if heads else "") != SCALAR_LOAD_HELPER:
+                        problems.append("%s:%d: %s outside %s()" % (name, line, op, SCALAR_LOAD_HELPER[1]))
+    if problems:
+        raise RuntimeError("inline asm may not issue loads the compiler does not track:\n" + "\n".join(problems))
+    return len(files)
 
 
 def kernel_resources(asm):
@@ -131,7 +214,15 @@ def check_hot_kernels(res):
 
 def build(verbose=False):
     sys.path.insert(0, HERE)
-    from isa_checks import check_forbidden  # a checker for the build machine only
+    try:
+        from isa_checks import check_forbidden  # travels with the sources on the build machine only
+    except ImportError:
+        print("build: isa_checks.py is not here, the scan for forbidden instructions is skipped "
+              "(the inline-asm, scalar-prefetch and spill checks still run)", file=sys.stderr)
+
+        def check_forbidden(text, where=""):
+            return None
+    check_asm_sources()
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = []
     procs = []
@@ -159,18 +250,22 @@ def build(verbose=False):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if verbose and out.strip():
             print(out)
-    asm = None
+    asm, n = None, 0
     for src, p in listings:
         text, _ = p.communicate()
         if p.returncode != 0:
             raise RuntimeError("hipcc -S failed on %s" % src)
-        check_forbidden(text, os.path.basename(src))  # isa_checks.py, imported below
+        check_forbidden(text, os.path.basename(src))
+        # ISA-level safety checks, every kernel of every source: no untracked load from inline asm, and no
+        # instruction touches an SGPR whose scalar load is still in flight
+        prefetchers = check_inline_asm_loads(text, os.path.basename(src))
+        n += check_scalar_prefetch(text)
         if os.path.basename(src) == "dense.hip":
             asm = text
-    # ISA-level safety check of the kernels that prefetch through inline-asm scalar loads
-    n = check_scalar_prefetch(asm)
+            if not any("dense_fwd_f32_pipe" in kname for kname in prefetchers):
+                raise RuntimeError("scalar-prefetch check found no pipelined forward kernel to verify")
     if n < 8:
-        raise RuntimeError("scalar-prefetch check found no pipelined forward kernel to verify")
+        raise RuntimeError("scalar-prefetch check verified only %d loads" % n)
     if verbose:
         print("scalar-prefetch check: %d loads verified" % n)
     res = kernel_resources(asm)

@@ -205,8 +205,77 @@ _ZN1_18dense_fwd_f32_pipeILi64EEEv: ; @k
             build.check_scalar_prefetch(bad)
     with pytest.raises(RuntimeError, match="in flight"):
         build.check_scalar_prefetch(good.replace("	s_waitcnt lgkmcnt(0)\n", ""))
-    # kernels without the prefetch idiom are not inspected
-    assert build.check_scalar_prefetch(good.replace("dense_fwd_f32_pipe", "other_kernel")) == 0
+    # every kernel of a listing is walked, whatever its name; a set of names narrows the walk
+    other = good.replace("dense_fwd_f32_pipe", "other_kernel")
+    assert build.check_scalar_prefetch(other) == 1
+    assert build.check_scalar_prefetch(other, {"_ZN1_18dense_fwd_f32_pipeILi64EEEv"}) == 0
+    with pytest.raises(RuntimeError, match="in flight"):
+        build.check_scalar_prefetch(other.replace("	v_subrev_f32_e32 v1, s4, v2", "	s_mov_b32 s36, s2"))
+
+
+def test_build_rejects_untracked_loads_in_inline_asm():
+    """Loads whose result arrives later may not be issued from inline asm, in any kernel of any source: the
+    compiler does not know the destination registers are still being written (a launch built that way took a GPU
+    memory fault).  Checked on the listing (between the compiler's ASMSTART/ASMEND marks) and on the sources;
+    scalar loads are allowed in the one helper and then verified instruction by instruction."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import build
+    listing = """
+_Z5kern1v: ; @k
+	buffer_load_dword v1, v0, s[0:3], 0 offen
+	;;#ASMSTART
+	v_fmac_f32 v1, v2, v3
+	;;#ASMEND
+	s_endpgm
+_Z5kern2v: ; @k
+	;;#ASMSTART
+	s_load_dwordx16 s[36:51], s[0:1], 0x0
+	;;#ASMEND
+	;;#ASMSTART
+	s_waitcnt lgkmcnt(0)
+	;;#ASMEND
+	s_endpgm
+"""
+    assert build.check_inline_asm_loads(listing) == {"_Z5kern2v"}
+    for bad in ("buffer_load_dword v4, v0, s[0:3], 0 offen", "global_load_dwordx4 v[4:7], v[0:1], off",
+                "flat_load_dword v4, v[0:1]", "ds_read_b128 v[4:7], v0", "scratch_load_dword v4, off, s0",
+                "global_atomic_add_rtn_u32 v4, v[0:1], v2, off", "buffer_atomic_add_f32 v1, v0, s[0:3], 0 offen"):
+        with pytest.raises(RuntimeError, match="does not track"):
+            build.check_inline_asm_loads(listing.replace("	v_fmac_f32 v1, v2, v3", "	" + bad), "x.hip")
+    # the shipped sources obey the rule; a second scalar-load site, or a vector load, in any file does not
+    assert build.check_asm_sources() >= 10
+    ok = {"dense.hip": 'void sload32(int& a, const float* p)\n{\n\tasm volatile("s_load_dword %0, %1, 0x0" : "=&s"(a) : "s"(p));\n}\n'}
+    assert build.check_asm_sources(ok) == 1
+    with pytest.raises(RuntimeError, match="outside sload32"):
+        build.check_asm_sources({"sparse.hip": ok["dense.hip"]})
+    with pytest.raises(RuntimeError, match="outside sload32"):
+        build.check_asm_sources({"dense.hip": ok["dense.hip"].replace("sload32", "other")})
+    with pytest.raises(RuntimeError, match="issues buffer_load_dword"):
+        build.check_asm_sources({"dense.hip": 'void f()\n{\n\tasm volatile("v_nop\\n\\tbuffer_load_dword %0, %1, %2, 0 offen" : "=v"(x) : "v"(o), "s"(r));\n}\n'})
+    with pytest.raises(RuntimeError, match="issues ds_read_b32"):
+        build.check_asm_sources({"fused.hip": 'void f()\n{\n\tasm("ds_read_b32 %0, %1" : "=v"(x) : "v"(o));\n}\n'})
+
+
+def test_build_runs_where_the_forbidden_instruction_list_does_not_travel(monkeypatch, capsys):
+    """isa_checks.py names instructions and stays on the build machine; build() must still import and run its
+    other checks without it.  hipcc is replaced by a stand-in that fails at once, so only the start is walked."""
+    import builtins
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import build
+    real_import = builtins.__import__
+
+    def no_isa_checks(name, *a, **kw):
+        if name == "isa_checks":
+            raise ImportError("No module named 'isa_checks'")
+        return real_import(name, *a, **kw)
+    monkeypatch.delitem(sys.modules, "isa_checks", raising=False)
+    monkeypatch.setattr(builtins, "__import__", no_isa_checks)
+    monkeypatch.setenv("HIPCC", "/bin/false")
+    with pytest.raises(RuntimeError, match="hipcc failed"):
+        build.build()
+    assert "forbidden instructions is skipped" in capsys.readouterr().err
 
 
 def test_build_rejects_spills_in_the_hot_kernels():
@@ -295,6 +364,20 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
     q, k = torch.zeros(B, T, H, W), torch.zeros(B, T, H, W)
     v, vb = torch.zeros(B, T, H, Wv), torch.zeros(B, T, H, Wv)
     coo = torch.zeros(E, 4, dtype=torch.int32)
+    # paths that have not passed on a GPU yet are closed unless asked for by name
+    monkeypatch.setattr(drv, "_enabled", set())
+    with pytest.raises(RuntimeError, match="experimental"):
+        drv.dense_fused_forward(q, k, v)
+    with pytest.raises(RuntimeError, match="experimental"):
+        drv.dense_forward_fixed(q, k)
+    with pytest.raises(RuntimeError, match="experimental.*rows16"):
+        drv.sparse_forward(v.half(), q.half(), k.half(), coo, 3, True)
+    with pytest.raises(RuntimeError, match="experimental.*rows16"):
+        drv.bidi_backward(v.bfloat16(), v.bfloat16(), vb.bfloat16(), q.bfloat16(), k.bfloat16(), coo,
+                          torch.zeros(B, E, H), 3, True)
+    with pytest.raises(ValueError, match="unknown experimental"):
+        drv.enable_experimental("everything")
+    assert drv.enable_experimental("rows16", "fused", "fixed") == frozenset(drv.EXPERIMENTAL)
     a, = drv.dense_forward(q, k)
     assert a.shape == (B, T, T, H)
     dq, dk = drv.dense_backward(torch.zeros(B, T, T, H), q, k)
@@ -372,6 +455,7 @@ def test_operator_modules_autograd_plumbing_without_a_gpu(monkeypatch):
     monkeypatch.setattr(drv, "check_input", lambda x, name: None)
     monkeypatch.setattr(drv, "stream_of", lambda x: None)
     monkeypatch.setattr(torch.cuda, "device", lambda d: contextlib.nullcontext())
+    monkeypatch.setattr(drv, "_enabled", {"fused"})
     B, T, H, W, E = 2, 5, 3, 8, 6
     mk = lambda *s: torch.zeros(*s, requires_grad=True)
     q, k = mk(B, T, H, W), mk(B, T, H, W)

@@ -22,6 +22,13 @@ from oracle import oracle
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True, scope="module")
+def _opt_in():
+    """These paths stay closed to the public operators until this file has passed on a GPU."""
+    import _l1attn_hip as drv
+    drv.enable_experimental("fused", "fixed")
+
 F32_TOL, F64_TOL = 1e-5, 1e-12
 
 

@@ -26,6 +26,13 @@ from oracle import oracle
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True, scope="module")
+def _opt_in():
+    """These paths stay closed to the public operators until this file has passed on a GPU."""
+    import _l1attn_hip as drv
+    drv.enable_experimental("rows16")
+
 TOL = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}
 DTYPES = [torch.float16, torch.bfloat16]
 
