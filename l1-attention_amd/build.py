@@ -1,6 +1,7 @@
-"""Compile the HIP sources under csrc/ into libl1attn_hip.so next to this file.
+"""Compile the HIP sources under csrc/ into libl1attn_hip.so, and the host-CPU twin under csrc_cpu/ into
+libl1attn_cpu.so, next to this file.
 
-    python build.py            # hipcc --offload-arch=gfx950, in-tree output
+    python build.py            # hipcc --offload-arch=gfx950 and g++, in-tree output
 
 hipcc cross-compiles without a GPU.  Packed fp32 instructions are disabled for all device
 code (-packed-fp32-ops): the kernels issue scalar-per-lane fp32 VALU operations only.
@@ -13,6 +14,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libl1attn_hip.so")
+CPU_LIB = os.path.join(HERE, "libl1attn_cpu.so")
 ARCH = "gfx950"
 
 
@@ -280,5 +282,37 @@ def build(verbose=False):
     return LIB
 
 
+def build_cpu(verbose=False):
+    """libl1attn_cpu.so: the API file once, the kernels twice (baseline x86-64 and AVX2 + FMA; the library picks
+    the copy the processor supports when it is loaded)."""
+    cxx = os.environ.get("CXX", "g++")
+    src = os.path.join(HERE, "csrc_cpu")
+    out = os.path.join(HERE, "build")
+    os.makedirs(out, exist_ok=True)
+    common = [cxx, "-O3", "-std=c++17", "-fPIC", "-fopenmp", "-fno-fast-math", "-Wall"]
+    jobs = [
+        (common + ["-c", os.path.join(src, "l1attn_cpu.cpp")], "l1attn_cpu.o"),
+        (common + ["-ffp-contract=off", "-DL1CPU_NS=l1cpu_generic", "-c", os.path.join(src, "l1attn_cpu_kernels.cpp")],
+         "l1attn_cpu_kernels_generic.o"),
+        (common + ["-mavx2", "-mfma", "-DL1CPU_NS=l1cpu_avx2", "-c", os.path.join(src, "l1attn_cpu_kernels.cpp")],
+         "l1attn_cpu_kernels_avx2.o"),
+    ]
+    procs = []
+    for cmd, obj in jobs:
+        cmd = cmd + ["-o", os.path.join(out, obj)]
+        if verbose:
+            print(" ".join(cmd))
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for cmd, p in procs:
+        text, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError("%s failed:\n%s" % (" ".join(cmd), text))
+        if verbose and text.strip():
+            print(text)
+    subprocess.run([cxx, "-shared", "-fopenmp", "-o", CPU_LIB] + [os.path.join(out, obj) for _, obj in jobs], check=True)
+    return CPU_LIB
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    print(build_cpu(verbose="-v" in sys.argv))

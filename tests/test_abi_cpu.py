@@ -483,3 +483,43 @@ def test_operator_modules_autograd_plumbing_without_a_gpu(monkeypatch):
     assert all(t.grad is not None and t.grad.shape == t.shape for t in (q, k, v))
     assert [c for c in _FakeLib.calls if not c.endswith("_bytes")] == \
         ["l1attn_fused_fwd_f32", "l1attn_fused_bwd_stage_f32", "l1attn_dense_bwd_f32"]
+
+
+def test_native_module_stand_ins_without_a_gpu(monkeypatch):
+    """The three modules named like the reference's pybind11 drivers (cuda/l1attn_cuda_drv.cpp:106-109,
+    cuda/l1attn_sparse_cuda_drv.cpp:71-74, cuda/l1attn_sparse_bidi_cuda_drv.cpp:77-80): forward/backward with the
+    reference's argument order and list returns, called the way the reference's own autograd Functions call them
+    (saved dst_mxlen / use_softmax come back as .item() values: cuda/l1attn_sparse_cuda.py:16, :42-46)."""
+    import contextlib
+    import sys
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import _l1attn_hip as drv
+    import l1attn_cuda_drv, l1attn_sparse_cuda_drv, l1attn_sparse_bidi_cuda_drv
+    for m in (l1attn_cuda_drv, l1attn_sparse_cuda_drv, l1attn_sparse_bidi_cuda_drv):
+        assert callable(m.forward) and callable(m.backward)
+    q = torch.randn(1, 4, 2, 8)
+    with pytest.raises(RuntimeError, match="q must be a CUDA tensor"):      # CHECK_INPUT, library not needed
+        l1attn_cuda_drv.forward(q, q)
+    with pytest.raises(RuntimeError, match="v must be a CUDA tensor"):
+        l1attn_sparse_cuda_drv.forward(q, q, q, torch.zeros(3, 4, dtype=torch.int32), 2, True)
+    with pytest.raises(RuntimeError, match="dvo must be a CUDA tensor"):
+        l1attn_sparse_bidi_cuda_drv.backward(q, q, q, q, q, torch.zeros(3, 4, dtype=torch.int32), q, 2, True)
+    monkeypatch.setattr(drv, "lib", lambda: _FakeLib())
+    monkeypatch.setattr(drv, "check_input", lambda x, name: None)
+    monkeypatch.setattr(drv, "stream_of", lambda x: None)
+    monkeypatch.setattr(torch.cuda, "device", lambda d: contextlib.nullcontext())
+    B, T, H, W, E = 2, 5, 3, 8, 6
+    q, k, v, vb = (torch.zeros(B, T, H, W) for _ in range(4))
+    coo = torch.zeros(E, 4, dtype=torch.int32)
+    attn = l1attn_cuda_drv.forward(q, k)
+    assert isinstance(attn, list) and attn[0].shape == (B, T, T, H)
+    d_q, d_k = l1attn_cuda_drv.backward(torch.zeros(B, T, T, H), q, k)
+    assert d_q.shape == q.shape and d_k.shape == k.shape
+    dmx, sm = torch.tensor(3), torch.tensor(True)
+    vo, attn = l1attn_sparse_cuda_drv.forward(v, q, k, coo, 3, True)
+    d_v, d_q, d_k = l1attn_sparse_cuda_drv.backward(torch.zeros_like(vo), v, q, k, coo, attn, dmx.item(), sm.item())
+    assert vo.shape == v.shape and [g.shape for g in (d_v, d_q, d_k)] == [v.shape, q.shape, k.shape]
+    vo, attn = l1attn_sparse_bidi_cuda_drv.forward(v, vb, q, k, coo, 3, False)
+    grads = l1attn_sparse_bidi_cuda_drv.backward(torch.zeros_like(vo), v, vb, q, k, coo, attn, dmx.item(), False)
+    assert len(grads) == 4 and all(g.shape == v.shape for g in grads)
