@@ -49,6 +49,9 @@ def _walk_kernels(asm_text):
         if l.startswith("_Z") and ":" in l.split(";")[0]:
             cur, in_asm = l.split(":")[0], False
             continue
+        if l.startswith(".Lfunc_end"):  # what follows the last function of a listing is metadata, not code
+            cur = None
+            continue
         if cur is None or not l or l[0] in ";.":
             continue
         l = l.split(";")[0].strip()
@@ -79,16 +82,15 @@ def check_inline_asm_loads(asm_text, where=""):
 
 
 def check_scalar_prefetch(asm_text, kernels=None):
-    """Static check of the scalar loads in the generated ISA, meant for the kernels that issue them from
-    inline asm and cheap enough to run on every kernel.
+    """Static check of the scalar loads in the generated ISA of the kernels that issue them from inline asm.
 
     The pipelined forward kernels issue `s_load_dwordx16` from inline asm and wait for it one chunk of math later.
     The compiler does not know that the destination SGPRs are written asynchronously: if register
     pressure makes it spill, copy or reuse them between the load and the next `s_waitcnt lgkmcnt(0)`,
     the late-arriving data lands in whatever lives there by then (a pointer, an exec mask) and the
-    kernel faults.  This walks the kernels (`kernels`: a set of mangled names, default: every kernel of the
-    listing; straight-line order, which is how both the compiler and the helper lay loads and waits out) and
-    fails the build if any instruction reads or
+    kernel faults.  This walks the kernels in `kernels` (a set of mangled names: build() passes every kernel
+    whose inline asm issues a scalar load, whatever its name or source file; None walks all, which only suits
+    straight-line listings since the walk does not follow branches) and fails the build if any instruction reads or
     writes an SGPR that still has a scalar load in flight, or if the kernel ends with one in flight.
     Returns the number of scalar loads checked."""
     cur, inflight, n_loads, problems = None, set(), 0, []
@@ -159,6 +161,21 @@ def check_asm_sources(files=None):
     if problems:
         raise RuntimeError("inline asm may not issue loads the compiler does not track:\n" + "\n".join(problems))
     return len(files)
+
+
+def isa_digests(asm_text):
+    """{kernel: (sha256 of its instruction stream, number of instructions)} for a device listing: the instructions
+    with their operands, in order, without comments, labels and directives.  Two builds whose digests agree run
+    the same machine code for that kernel."""
+    import hashlib
+    streams = {}
+    for kern, _, l, _ in _walk_kernels(asm_text):
+        if re.match(r"^[\w.$]+:$", l):  # a label
+            continue
+        # branch targets carry the function's ordinal in the file (.LBB<ordinal>_<block>): drop the ordinal, so
+        # that adding a kernel to a source does not change the digests of the others
+        streams.setdefault(kern, []).append(re.sub(r"\.LBB\d+_", ".LBB_", " ".join(l.split())))
+    return {k: (hashlib.sha256("\n".join(v).encode()).hexdigest()[:16], len(v)) for k, v in streams.items()}
 
 
 def kernel_resources(asm):
@@ -252,16 +269,18 @@ def build(verbose=False):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if verbose and out.strip():
             print(out)
-    asm, n = None, 0
+    asm, n, digests = None, 0, []
     for src, p in listings:
         text, _ = p.communicate()
         if p.returncode != 0:
             raise RuntimeError("hipcc -S failed on %s" % src)
         check_forbidden(text, os.path.basename(src))
-        # ISA-level safety checks, every kernel of every source: no untracked load from inline asm, and no
-        # instruction touches an SGPR whose scalar load is still in flight
+        # ISA-level safety checks, every kernel of every source: no untracked load from inline asm, and in
+        # every kernel whose inline asm issues scalar loads no instruction touches an SGPR still in flight
         prefetchers = check_inline_asm_loads(text, os.path.basename(src))
-        n += check_scalar_prefetch(text)
+        n += check_scalar_prefetch(text, prefetchers)
+        for kname, (h, cnt) in sorted(isa_digests(text).items()):
+            digests.append("%s %s %s %d" % (os.path.basename(src), kname, h, cnt))
         if os.path.basename(src) == "dense.hip":
             asm = text
             if not any("dense_fwd_f32_pipe" in kname for kname in prefetchers):
@@ -275,6 +294,10 @@ def build(verbose=False):
     with open(os.path.join(HERE, "build", "dense_kernel_resources.txt"), "w") as f:
         for name in sorted(res):
             f.write("%s %s\n" % (name, " ".join("%s=%d" % kv for kv in sorted(res[name].items()))))
+    # one line per kernel: source, mangled name, digest of its instruction stream, instruction count.  Kept under
+    # version control, so that the history shows which commits changed which kernel's machine code.
+    with open(os.path.join(HERE, "isa_digests.txt"), "w") as f:
+        f.write("\n".join(digests) + "\n")
     cmd = [hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd))
