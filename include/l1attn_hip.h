@@ -71,8 +71,10 @@ int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn,
  * held in `workspace` (device memory, 256-byte aligned, at least
  * l1attn_dense_bwd_workspace_bytes() for full speed; any multiple of one batch's share works,
  * the batches are then processed in several launches).  The f64 entry needs no workspace.
- * f32 fast path: sign() is taken from (q-k)*2^64, exact for |q|,|k| < 2^63 and differences
- * that are 0 or at least 2^-64 in magnitude.  For 2048 <= T <= 8192 (and enough work to fill
+ * f32 tiled path (T >= 16 and H*W >= 32): sign() is taken as clamp(q*2^64 - k*2^64, -1, 1), exact for
+ * |q|,|k| < 2^63 and differences that are 0 or at least 2^-64 in magnitude; a smaller non-zero
+ * difference d enters with weight d*2^64 instead of +-1, larger magnitudes overflow (unspecified
+ * result).  The generic f32 kernels (smaller shapes) and the f64 entry compare exactly.  For 2048 <= T <= 8192 (and enough work to fill
  * the GPU) sign() is taken from the column ranks of l1attn_dense_column_ranks_f32 instead, exact
  * for all finite inputs; the gradient is then assembled as 2*sum(hv*d_attn) - sum(d_attn) with
  * hv = (sign+1)/2, so an element whose pairs all tie comes out as a rounding residue of the two
