@@ -429,7 +429,23 @@ def cpu_baseline():
     oracle.dense_bwd(dA32, q32, k32)
     dt_mt = time.perf_counter() - t0
     oracle.set_threads(1)
+    # this repository's own CPU operator package (l1attn_cpp over libl1attn_cpu.so; product code, not the baseline)
+    pkg = None
+    try:
+        import _l1attn_cpu
+        _l1attn_cpu.set_threads(ncores)
+        _l1attn_cpu.dense_forward(q32, k32)
+        t0 = time.perf_counter()
+        _l1attn_cpu.dense_forward(q32, k32)
+        _l1attn_cpu.dense_backward(dA32, q32, k32)
+        dt_pkg = time.perf_counter() - t0
+        _l1attn_cpu.set_threads(0)
+        pkg = {"value": 6 * N / dt_pkg / 1e9, "unit": "GOP/s", "cores": ncores,
+               "note": "l1attn_cpp (the CPU twin of the operators, fp32, OpenMP), same sample"}
+    except Exception as e:
+        log("CPU operator package not timed:", repr(e))
     return {
+        "cpu_operator_package_fp32": pkg,
         "value": 6 * N / dt / 1e9, "unit": "GOP/s", "cores": 1, "kind": kind,
         "sample": "dense fwd+bwd fp64, B=1 T=1024 H=16 W=64 (1/128 of the headline pair-elements), %.1f s" % dt,
         "port_fp32_openmp": {"value": 6 * N / dt_mt / 1e9, "unit": "GOP/s", "cores": ncores,
