@@ -147,6 +147,14 @@ int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* 
                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
 int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, double* vo, double* lse,
                          int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
+/*
+ * The f32 fused forward with the k and v rows streamed through a software pipeline of scalar loads (the
+ * technique of the dense forward) for W == Wv in {32, 64}; every other shape runs what l1attn_fused_fwd_f32
+ * runs.  Same arithmetic in the same order: results equal l1attn_fused_fwd_f32's bit for bit.  Kept as an entry of
+ * its own until both have been timed on a GPU.  No counterpart in the reference.
+ */
+int l1attn_fused_fwd_pipe_f32(const float* q, const float* k, const float* v, float* vo, float* lse,
+                              int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
 
 /*
  * Backward of the fused forward, first stage.  With p[s,t] = exp(a[s,t] - lse[t]), dp[s,t] = v[s].dvo[t],

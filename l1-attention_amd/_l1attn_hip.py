@@ -89,6 +89,9 @@ def lib():
             f = getattr(L, "l1attn_fused_fwd_" + sfx)
             f.restype = _c_i
             f.argtypes = [_c_p] * 5 + [_c_i64] * 5 + [_c_p]
+            if sfx == "f32":
+                L.l1attn_fused_fwd_pipe_f32.restype = _c_i
+                L.l1attn_fused_fwd_pipe_f32.argtypes = f.argtypes
             f = getattr(L, "l1attn_fused_bwd_stage_" + sfx)
             f.restype = _c_i
             f.argtypes = [_c_p] * 8 + [_c_i64] * 5 + [_c_p]
@@ -238,11 +241,13 @@ def dense_backward(d_attn, q, k):
     return [dq, dk]
 
 
-def dense_fused_forward(q, k, v, want_lse=False):
+def dense_fused_forward(q, k, v, want_lse=False, pipelined=False):
     """Fused forward: vo[b,t,h,:] = sum_s p[s] * v[b,s,h,:] with p the softmax over src of the L1 logits
     and a no-op zero logit (1 + sum in the denominator), without materialising the [B,T,T,H] logits.
     What example-setfind/setfind.py:128-136 composes from L1Attn, softmax and einsum.
-    Returns [vo, lse]; lse [B,T,H] = log(1 + sum_s exp(a)) if want_lse else None."""
+    Returns [vo, lse]; lse [B,T,H] = log(1 + sum_s exp(a)) if want_lse else None.
+    pipelined (float32 only): the entry whose kernels stream k and v through a software pipeline of scalar loads;
+    same results bit for bit."""
     _require_experimental("fused", "the fused L1 attention operator")
     for x, n in ((q, "q"), (k, "k"), (v, "v")):
         check_input(x, n)
@@ -256,9 +261,10 @@ def dense_fused_forward(q, k, v, want_lse=False):
     vo = torch.empty_like(v)
     lse = torch.empty((B, T, H), dtype=q.dtype, device=q.device) if want_lse else None
     with torch.cuda.device(q.device):
-        rc = getattr(lib(), "l1attn_fused_fwd_" + sfx)(
+        name = "l1attn_fused_fwd_pipe_f32" if (pipelined and sfx == "f32") else "l1attn_fused_fwd_" + sfx
+        rc = getattr(lib(), name)(
             ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse) if lse is not None else None, B, T, H, W, Wv, stream_of(q))
-    check(rc, "l1attn_fused_fwd_" + sfx)
+    check(rc, name)
     return [vo, lse]
 
 

@@ -127,7 +127,7 @@ def check_scalar_prefetch(asm_text, kernels=None):
 
 
 _ASM_STMT = re.compile(r"\basm\s*(?:volatile\s*)?\(")
-SCALAR_LOAD_HELPER = ("dense.hip", "sload32")  # the one function whose inline asm may issue scalar loads
+SCALAR_LOAD_HELPER = ("sload.h", "sload32")  # the one function whose inline asm may issue scalar loads
 
 
 def check_asm_sources(files=None):

@@ -24,6 +24,7 @@
 // Generic kernels (any shape, float or double, exact comparisons) cover everything else.
 #include "common.h"
 #include "dense_rank.h"
+#include "sload.h"
 #include "xcd.h"
 #include "fixed.h"
 #include <math.h>
@@ -212,18 +213,6 @@ __global__ __launch_bounds__(1024) void dense_fwd_f32_fast(const float* __restri
 // chunk c+1 is issued before the 64 VALU instructions of chunk c, so one chunk of compute (times the
 // waves interleaved on the SIMD) covers the latency.  Scalar loads return out of order, hence the
 // only wait used is lgkmcnt(0).
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-__device__ __forceinline__ void sload32(f32x16& lo, f32x16& hi, const float* p)
-{
-	// early-clobber outputs: the second load must still see the pointer
-	asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40" : "=&s"(lo), "=&s"(hi) : "s"(p));
-}
-__device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
-{
-	asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(lo), "+s"(hi));
-}
-
 // FIXED: q and k hold biased fixed-point values (32-bit unsigned, see fixed_quantise) on a grid of gq[b*H+h]
 // per (batch, head); the pair-element is then one v_sad_u32 (|a - b| + c on unsigned integers) instead of
 // v_sub + v_add |x|, the sum of W <= 64 terms is exact and at most 2^31, and the logit is sum * grid * scale.

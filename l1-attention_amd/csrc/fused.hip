@@ -1,4 +1,4 @@
-// Fused dense L1 attention for gfx950, forward only: logits, softmax over the src tokens with the
+// Fused dense L1 attention for gfx950: logits, softmax over the src tokens with the
 // "no-op" zero logit, and the value sum, without ever writing the [B,T,T,H] logits:
 //
 //   a[s]        = -1/sqrt(W) * sum_w |q[b,t,h,w] - k[b,s,h,w]|
@@ -17,6 +17,7 @@
 // and one v_fmac for the value sum; one exp per (src, dst, head).  No LDS, no atomics; src tokens are
 // summed in ascending order, so results repeat bit for bit.
 #include "common.h"
+#include "sload.h"
 #include "xcd.h"
 #include <math.h>
 
@@ -101,6 +102,103 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restric
 		kp += row;
 		vp += row;
 	}
+	if (store) {
+		const float inv = 1.0f / (1.0f + den);
+		float4* op = reinterpret_cast<float4*>(vo + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++)
+			op[w4] = make_float4(acc[w4 * 4 + 0] * inv, acc[w4 * 4 + 1] * inv, acc[w4 * 4 + 2] * inv,
+			                     acc[w4 * 4 + 3] * inv);
+		if (lse) lse[((int64_t)b * Tn + t) * H + h] = log1pf(den);
+	}
+}
+
+// Software-pipelined variant of the tiled forward for W == WV a multiple of 32: the same mapping and the same
+// arithmetic in the same order, but the k and v rows stream through two 32-float SGPR buffers (sload.h) as one
+// sequence of chunks -- k chunks of src token s, v chunks of s, k chunks of s + 1, ... -- with the load of the
+// next chunk issued before the VALU work on the current one.  A row holds an even number of chunks (2*W/32), so a
+// chunk's buffer is fixed by its place in the row.  The load issued after a row's last chunk is the first k chunk
+// of the next row, clamped to the last row at the end (read, never used), and drained after the loop.
+template <int W>
+__global__ __launch_bounds__(256) void fused_fwd_f32_pipe(const float* __restrict__ q, const float* __restrict__ k,
+                                                            const float* __restrict__ v, float* __restrict__ vo,
+                                                            float* __restrict__ lse, int Tn, int H, int n_hg, int NH,
+                                                            float scale)
+{
+	static_assert(W % 32 == 0, "whole 32-float chunks");
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.y / n_hg, hg = lb.y % n_hg;
+	const int h_raw = hg * NH + wave;
+	const int h = min(h_raw, H - 1);  // surplus waves of the last group redo head H-1 and store nothing
+	const int t_raw = lb.x * 64 + lane;
+	const int t = min(t_raw, Tn - 1);  // surplus lanes of the last tile redo token Tn-1 and store nothing
+	const bool store = h_raw < H && t_raw < Tn;
+
+	float qr[W], acc[W];
+	{
+		const float4* qp = reinterpret_cast<const float4*>(q + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = qp[w4];
+			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
+		}
+#pragma unroll
+		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+	}
+	float den = 0.0f;
+	constexpr int CPR = W / 32;  // chunks per k row and per v row
+	const int64_t row = (int64_t)H * W;
+	const float* const kb = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;  // src token 0 of this (b,h): wave-uniform
+	const float* const vb = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	f32x16 b0l, b0h, b1l, b1h;
+	sload32(b0l, b0h, kb);
+	__builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+	for (int s = 0; s < Tn; s++) {
+		const float* const krow = kb + s * row;
+		const float* const vrow = vb + s * row;
+		const float* const knext = kb + min(s + 1, Tn - 1) * row;
+		float a = 0.0f, p = 0.0f;
+#pragma unroll
+		for (int c = 0; c < 2 * CPR; c++) {
+			// the chunk after this one: the rest of the k row, then the v row, then the next token's k row
+			const float* const nxt = c + 1 < CPR ? krow + (c + 1) * 32 : c + 1 < 2 * CPR ? vrow + (c + 1 - CPR) * 32 : knext;
+			// (the scheduler may not move the previous chunk's VALU work below this chunk's wait: the wait would
+			// then come a few instructions after the load it waits for)
+			__builtin_amdgcn_sched_barrier(0);
+			if ((c & 1) == 0) {
+				swait32(b0l, b0h);
+				__builtin_amdgcn_sched_barrier(0);
+				sload32(b1l, b1h, nxt);
+				__builtin_amdgcn_sched_barrier(0);
+			} else {
+				swait32(b1l, b1h);
+				__builtin_amdgcn_sched_barrier(0);
+				sload32(b0l, b0h, nxt);
+				__builtin_amdgcn_sched_barrier(0);
+			}
+			const f32x16& lo = (c & 1) == 0 ? b0l : b1l;
+			const f32x16& hi = (c & 1) == 0 ? b0h : b1h;
+			if (c < CPR) {
+#pragma unroll
+				for (int i = 0; i < 16; i++) a += fabsf(qr[c * 32 + i] - lo[i]);
+#pragma unroll
+				for (int i = 0; i < 16; i++) a += fabsf(qr[c * 32 + 16 + i] - hi[i]);
+			} else {
+				if (c == CPR) {
+					p = expf(a * scale);
+					den += p;
+				}
+#pragma unroll
+				for (int i = 0; i < 16; i++) acc[(c - CPR) * 32 + i] += p * lo[i];
+#pragma unroll
+				for (int i = 0; i < 16; i++) acc[(c - CPR) * 32 + 16 + i] += p * hi[i];
+			}
+		}
+	}
+	swait32(b0l, b0h);  // drain the last prefetch before the wave ends
 	if (store) {
 		const float inv = 1.0f / (1.0f + den);
 		float4* op = reinterpret_cast<float4*>(vo + (((int64_t)b * Tn + t) * H + h) * (int64_t)W);
@@ -326,8 +424,10 @@ int launch_bwd_generic(const T* dvo, const T* q, const T* k, const T* v, const T
 
 extern "C" {
 
-int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse, int64_t B, int64_t T,
-                         int64_t H, int64_t W, int64_t Wv, void* stream)
+// pipe: take the software-pipelined kernel where it exists (W == Wv in {32, 64}); every other shape runs
+// what l1attn_fused_fwd_f32 runs
+static int fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse, int64_t B, int64_t T,
+                         int64_t H, int64_t W, int64_t Wv, void* stream, bool pipe)
 {
 	if (!shape_ok(B, T, H, W, Wv)) return L1ATTN_ERR_ARG;
 	if (B * T * H == 0) return L1ATTN_OK;
@@ -341,22 +441,37 @@ int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* 
 	if (!tiled) return launch_generic<float>(q, k, v, vo, lse, B, T, H, W, Wv, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
 	const dim3 grid((unsigned)l1_cdiv(T, 64), (unsigned)(B * n_hg), 1), block(64 * NH);
-#define L1_FUSED_CASE(WV)                                                                                        \
-	case WV:                                                                                                     \
-		hipLaunchKernelGGL(fused_fwd_f32_tile<WV>, grid, block, 0, st, q, k, v, vo, lse, (int)T, (int)H, (int)n_hg, \
-		                   NH, scale);                                                                           \
-		break
+#define L1_FUSED_CASE(KERNEL, WV)                                                                                \
+	hipLaunchKernelGGL(KERNEL<WV>, grid, block, 0, st, q, k, v, vo, lse, (int)T, (int)H, (int)n_hg, NH, scale)
 	switch (W) {
-		L1_FUSED_CASE(16);
-		L1_FUSED_CASE(32);
-		L1_FUSED_CASE(48);
-		L1_FUSED_CASE(64);
-		L1_FUSED_CASE(96);
+	case 16: L1_FUSED_CASE(fused_fwd_f32_tile, 16); break;
+	case 32:
+		if (pipe) L1_FUSED_CASE(fused_fwd_f32_pipe, 32);
+		else L1_FUSED_CASE(fused_fwd_f32_tile, 32);
+		break;
+	case 48: L1_FUSED_CASE(fused_fwd_f32_tile, 48); break;
+	case 64:
+		if (pipe) L1_FUSED_CASE(fused_fwd_f32_pipe, 64);
+		else L1_FUSED_CASE(fused_fwd_f32_tile, 64);
+		break;
+	case 96: L1_FUSED_CASE(fused_fwd_f32_tile, 96); break;  // (pipelined, its SGPR buffers would spill)
 	default: return L1ATTN_ERR_ARG;
 	}
 #undef L1_FUSED_CASE
 	L1_LAUNCH_CHECK();
 	return L1ATTN_OK;
+}
+
+int l1attn_fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse, int64_t B, int64_t T,
+                         int64_t H, int64_t W, int64_t Wv, void* stream)
+{
+	return fused_fwd_f32(q, k, v, vo, lse, B, T, H, W, Wv, stream, false);
+}
+
+int l1attn_fused_fwd_pipe_f32(const float* q, const float* k, const float* v, float* vo, float* lse, int64_t B,
+                              int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream)
+{
+	return fused_fwd_f32(q, k, v, vo, lse, B, T, H, W, Wv, stream, true);
 }
 
 int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, double* vo, double* lse, int64_t B,

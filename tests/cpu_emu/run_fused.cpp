@@ -1,18 +1,54 @@
 // TEST INFRASTRUCTURE: runs l1attn_fused_fwd_f32 / _f64 of csrc/fused.hip, compiled for the host with
 // the stand-in header next to this file, on inputs read from a file, and writes vo and lse.
-//   run_fused <in> <out> <f32|f64> <misalign>
+//   run_fused <in> <out> <f32|f64> <misalign> [pipe]      (pipe: forward through l1attn_fused_fwd_pipe_f32)
 // in : int64 B,T,H,W,Wv then q,k [B,T,H,W], v [B,T,H,Wv] and dvo [B,T,H,Wv] in the chosen type
 // out: vo [B,T,H,Wv], lse [B,T,H], one int64 (threads the forward ran), then the backward's first stage on
 //      the forward's own vo and lse: dA [B,T,T,H], dv [B,T,H,Wv], one int64 (threads it ran)
 // Buffers are malloc'ed at their exact sizes, so AddressSanitizer reports any access outside them.
 // misalign = 1 offsets every buffer by one element (the library then has to take its generic kernel).
+#include "hip/hip_runtime.h"
+#include <atomic>
+#include <string.h>
+
+// Host stand-in for csrc/sload.h (the one header of the library whose inline asm issues loads), with the
+// property that matters kept: the data of a prefetch arrives at the WAIT, not at the load.  sload32 poisons its
+// two buffers and remembers the source; swait32 (lgkmcnt(0): everything outstanding) delivers all remembered
+// loads.  A kernel that reads a buffer before its wait computes on NaNs, one that forgets the final drain leaves
+// `outstanding` above zero: both show in the test.
+#define L1ATTN_SLOAD_H
+struct f32x16 {
+	float a[16];
+	float operator[](int i) const { return a[i]; }
+};
+namespace emu_sload {
+struct Pending { f32x16 *lo, *hi; const float* p; };
+inline thread_local std::vector<Pending> pending;
+inline std::atomic<long> outstanding{0};
+}
+static inline void sload32(f32x16& lo, f32x16& hi, const float* p)
+{
+	for (int i = 0; i < 16; i++) lo.a[i] = hi.a[i] = NAN;
+	emu_sload::pending.push_back({&lo, &hi, p});
+	emu_sload::outstanding++;
+}
+static inline void swait32(f32x16&, f32x16&)
+{
+	for (const auto& x : emu_sload::pending) {
+		memcpy(x.lo->a, x.p, 64);
+		memcpy(x.hi->a, x.p + 16, 64);
+		emu_sload::outstanding--;
+	}
+	emu_sload::pending.clear();
+}
+static inline void __builtin_amdgcn_sched_barrier(int) {}
+
 #include "../../l1-attention_amd/csrc/fused.hip"
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
 template <typename T>
-static int run(FILE* fi, FILE* fo, const int64_t* d, bool f32, int mis)
+static int run(FILE* fi, FILE* fo, const int64_t* d, bool f32, int mis, bool pipe)
 {
 	const int64_t B = d[0], Tn = d[1], H = d[2], W = d[3], Wv = d[4];
 	const size_t nq = (size_t)(B * Tn * H * W), nv = (size_t)(B * Tn * H * Wv), nl = (size_t)(B * Tn * H);
@@ -21,11 +57,14 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, bool f32, int mis)
 	if (fread(q, sizeof(T), nq, fi) != nq || fread(k, sizeof(T), nq, fi) != nq || fread(v, sizeof(T), nv, fi) != nv)
 		return 3;
 	int rc;
-	if (f32) rc = l1attn_fused_fwd_f32((const float*)q, (const float*)k, (const float*)v, (float*)vo, (float*)lse, B,
-	                                   Tn, H, W, Wv, nullptr);
+	if (f32 && pipe) rc = l1attn_fused_fwd_pipe_f32((const float*)q, (const float*)k, (const float*)v, (float*)vo,
+	                                                (float*)lse, B, Tn, H, W, Wv, nullptr);
+	else if (f32) rc = l1attn_fused_fwd_f32((const float*)q, (const float*)k, (const float*)v, (float*)vo, (float*)lse, B,
+	                                        Tn, H, W, Wv, nullptr);
 	else rc = l1attn_fused_fwd_f64((const double*)q, (const double*)k, (const double*)v, (double*)vo, (double*)lse,
 	                               B, Tn, H, W, Wv, nullptr);
 	if (rc) return 10 + (rc < 0 ? -rc : rc);
+	if (emu_sload::outstanding != 0) return 9;  // a wave ended with a scalar prefetch in flight
 	fwrite(vo, sizeof(T), nv, fo);
 	fwrite(lse, sizeof(T), nl, fo);
 	int64_t n = emu::n_threads_run;
@@ -52,7 +91,8 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, bool f32, int mis)
 
 int main(int argc, char** argv)
 {
-	if (argc != 5) return 2;
+	if (argc != 5 && argc != 6) return 2;
+	const bool pipe = argc == 6 && strcmp(argv[5], "pipe") == 0;
 	FILE* fi = fopen(argv[1], "rb");
 	FILE* fo = fopen(argv[2], "wb");
 	if (!fi || !fo) return 2;
@@ -60,7 +100,7 @@ int main(int argc, char** argv)
 	if (fread(d, sizeof(int64_t), 5, fi) != 5) return 3;
 	const bool f32 = strcmp(argv[3], "f32") == 0;
 	const int mis = atoi(argv[4]);
-	const int rc = f32 ? run<float>(fi, fo, d, true, mis) : run<double>(fi, fo, d, false, mis);
+	const int rc = f32 ? run<float>(fi, fo, d, true, mis, pipe) : run<double>(fi, fo, d, false, mis, pipe);
 	fclose(fi);
 	fclose(fo);
 	return rc;

@@ -245,12 +245,12 @@ _Z5kern2v: ; @k
             build.check_inline_asm_loads(listing.replace("	v_fmac_f32 v1, v2, v3", "	" + bad), "x.hip")
     # the shipped sources obey the rule; a second scalar-load site, or a vector load, in any file does not
     assert build.check_asm_sources() >= 10
-    ok = {"dense.hip": 'void sload32(int& a, const float* p)\n{\n\tasm volatile("s_load_dword %0, %1, 0x0" : "=&s"(a) : "s"(p));\n}\n'}
+    ok = {"sload.h": 'void sload32(int& a, const float* p)\n{\n\tasm volatile("s_load_dword %0, %1, 0x0" : "=&s"(a) : "s"(p));\n}\n'}
     assert build.check_asm_sources(ok) == 1
     with pytest.raises(RuntimeError, match="outside sload32"):
-        build.check_asm_sources({"sparse.hip": ok["dense.hip"]})
+        build.check_asm_sources({"sparse.hip": ok["sload.h"]})
     with pytest.raises(RuntimeError, match="outside sload32"):
-        build.check_asm_sources({"dense.hip": ok["dense.hip"].replace("sload32", "other")})
+        build.check_asm_sources({"sload.h": ok["sload.h"].replace("sload32", "other")})
     with pytest.raises(RuntimeError, match="issues buffer_load_dword"):
         build.check_asm_sources({"dense.hip": 'void f()\n{\n\tasm volatile("v_nop\\n\\tbuffer_load_dword %0, %1, %2, 0 offen" : "=v"(x) : "v"(o), "s"(r));\n}\n'})
     with pytest.raises(RuntimeError, match="issues ds_read_b32"):

@@ -41,7 +41,7 @@ def runner_tsan(tmp_path_factory):
     return exe
 
 
-def _run(exe, tmp_path, q, k, v, misalign=0):
+def _run(exe, tmp_path, q, k, v, misalign=0, pipe=False):
     """-> dict: vo, lse, threads (forward), dA, dv, bwd_threads (first stage of the backward on a seeded dvo),
     and dvo itself."""
     B, T, H, W = q.shape
@@ -54,7 +54,8 @@ def _run(exe, tmp_path, q, k, v, misalign=0):
         for x in (q, k, v, dvo):
             f.write(x.contiguous().numpy().tobytes())
     env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
-    r = subprocess.run([exe, fin, fout, kind, str(misalign)], env=env, capture_output=True, text=True)
+    r = subprocess.run([exe, fin, fout, kind, str(misalign)] + (["pipe"] if pipe else []), env=env,
+                       capture_output=True, text=True)
     assert r.returncode == 0, (r.returncode, r.stderr[-2000:])
     raw = open(fout, "rb").read()
     dt = np.float32 if kind == "f32" else np.float64
@@ -123,6 +124,28 @@ def test_fused_tiled_kernels_on_cpu(runner, tmp_path, shape):
     ref, ref_lse = _ref(q, k, v)
     assert cf.rel_err(r["vo"], ref) <= 1e-5 and cf.rel_err(r["lse"], ref_lse) <= 1e-5
     _check_backward(r, q, k, v, 1e-4)
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 4, 32), (1, 100, 3, 64), (2, 70, 6, 32), (1, 33, 9, 64), (1, 1000, 1, 32)])
+def test_fused_pipelined_forward_on_cpu(runner, tmp_path, shape):
+    """The software-pipelined forward (l1attn_fused_fwd_pipe_f32).  The host stand-in for the scalar prefetch
+    delivers a chunk's data at the wait and poisons the buffer at the load, so reading a buffer before its wait, a
+    chunk taken from the wrong buffer, a wrong chunk address or a missing final drain all fail here.  Same arithmetic
+    in the same order as the plain tiled kernel: equal bit for bit."""
+    B, T, H, W = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
+    plain = _run(runner, tmp_path, q, k, v)
+    piped = _run(runner, tmp_path, q, k, v, pipe=True)
+    NH = min(H, 4)
+    assert piped["threads"] == -(-T // 64) * B * -(-H // NH) * 64 * NH
+    assert torch.equal(piped["vo"], plain["vo"]) and torch.equal(piped["lse"], plain["lse"])
+    ref, ref_lse = _ref(q, k, v)
+    assert cf.rel_err(piped["vo"], ref) <= 1e-5 and cf.rel_err(piped["lse"], ref_lse) <= 1e-5
+    # widths without a pipelined kernel run what the plain entry runs
+    if shape == (2, 64, 4, 32):
+        q16, k16, v16 = q[..., :16].contiguous(), k[..., :16].contiguous(), v[..., :16].contiguous()
+        assert torch.equal(_run(runner, tmp_path, q16, k16, v16, pipe=True)["vo"], _run(runner, tmp_path, q16, k16, v16)["vo"])
 
 
 GENERIC = [
