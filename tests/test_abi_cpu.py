@@ -389,6 +389,10 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
     vo, lse = drv.dense_fused_forward(q, k, v, want_lse=True)
     assert vo.shape == v.shape and lse.shape == (B, T, H) and _FakeLib.calls[-1] == "l1attn_fused_fwd_f32"
     assert drv.dense_fused_forward(q.double(), k.double(), v.double())[1] is None
+    drv.dense_fused_forward(q, k, v, pipelined=True)
+    assert _FakeLib.calls[-1] == "l1attn_fused_fwd_pipe_f32"
+    drv.dense_fused_forward(q.double(), k.double(), v.double(), pipelined=True)   # float64 has one entry
+    assert _FakeLib.calls[-1] == "l1attn_fused_fwd_f64"
     with pytest.raises(RuntimeError, match="equal leading dims"):
         drv.dense_fused_forward(q, k, torch.zeros(B, T + 1, H, Wv))
     with pytest.raises(RuntimeError, match="share dtype"):

@@ -76,6 +76,26 @@ def test_fused_forward_vs_oracle(shape):
     assert cf.rel_err(lse64.cpu(), ref_lse) <= F64_TOL
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 4, 32), (1, 100, 3, 64), (2, 70, 6, 32), (1, 33, 9, 64), (2, 1024, 8, 64),
+                                   (1, 40, 2, 48)])
+def test_fused_pipelined_forward_equals_the_plain_one(shape):
+    """l1attn_fused_fwd_pipe_f32 (k and v rows through the scalar-load pipeline; widths 32 and 64, any other width
+    runs the plain kernels): the same arithmetic in the same order, so equal to l1attn_fused_fwd_f32 bit for bit,
+    and within tolerance of the oracle.  Run after the plain forward's tests have passed."""
+    B, T, H, W = shape
+    print("case fused pipelined", shape, flush=True)
+    import _l1attn_hip as drv
+    g = torch.Generator().manual_seed(sum(shape))
+    q, k, v = (torch.randn(B, T, H, W, generator=g).cuda() for _ in range(3))
+    vo, lse = drv.dense_fused_forward(q, k, v, want_lse=True)
+    vop, lsep = drv.dense_fused_forward(q, k, v, want_lse=True, pipelined=True)
+    torch.cuda.synchronize()
+    assert torch.equal(vop, vo) and torch.equal(lsep, lse)
+    if T <= 128:
+        ref, ref_lse = oracle.fused_fwd(q.cpu().double(), k.cpu().double(), v.cpu().double())
+        assert cf.rel_err(vop.cpu(), ref) <= F32_TOL and cf.rel_err(lsep.cpu(), ref_lse) <= F32_TOL
+
+
 def test_fused_forward_unaligned_views_take_the_generic_kernel():
     print("case fused unaligned", flush=True)
     import _l1attn_hip as drv
