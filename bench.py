@@ -454,6 +454,14 @@ def cpu_baseline():
     }
 
 
+def _guarded(fn):
+    try:
+        return fn()
+    except Exception as e:  # noqa: BLE001
+        log("side measurement failed:", repr(e))
+        return {"error": repr(e)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -529,16 +537,28 @@ def main():
                                "(BASELINE.json configs[2], the headline dense configuration)",
                    "B": 8, "T": 4096, "H": 16, "W": 64},
         "frac_of_fp32_valu_peak": d["frac_of_valu_peak"],
-        "valu_probe": valu_probe(),
+        "valu_probe": _guarded(valu_probe),
         "dense": d,
         "roofline": roof,
     }
+    # The headline figures above are complete; a failure in a side leg is reported inside the line instead of
+    # taking the line with it.
     if not args.skip_sparse:
         log("sparse configurations ...")
-        out["sparse"] = sparse_configs(args.skip_cpu, args.only)
+        try:
+            out["sparse"] = sparse_configs(args.skip_cpu, args.only)
+        except Exception as e:  # noqa: BLE001
+            import traceback
+            log(traceback.format_exc())
+            out["sparse"] = {"error": repr(e)}
     if not args.skip_cpu:
         log("cpu baseline ...")
-        out["cpu_baseline"] = cpu_baseline()
+        try:
+            out["cpu_baseline"] = cpu_baseline()
+        except Exception as e:  # noqa: BLE001
+            import traceback
+            log(traceback.format_exc())
+            out["cpu_baseline"] = {"error": repr(e)}
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out), flush=True)
