@@ -390,6 +390,38 @@ def valu_probe():
             "lane_tops": tops, "frac_of_nominal_peak": tops / P_VALU_TOPS, "ms": ms}
 
 
+def cpu_baseline_sparse(mods, ncores):
+    """Configuration 4 in full (B4 T4096 H8 W32, about 133 k edges) on the host: the reference's own CPU extension
+    (float64, one thread; its softmax Jacobian loop is O(dst_mxlen^2) per token and head) when oracle/_ref is
+    there, and this repository's CPU operator package (float32, all cores).  Forward + backward, edges per second."""
+    import torch
+    import workloads
+    import _l1attn_cpu
+    B, T, H, W = 4, 4096, 8, 32
+    co = workloads.uniform_degree_graph(T, 64, seed=1004)
+    coo, dmx, _ = _l1attn_cpu.expand_coo(co)
+    v, _, q, k = workloads.sparse_inputs(B, T, H, W, seed=1004, n=4)
+    dvo = torch.randn(B, T, H, W, generator=torch.Generator().manual_seed(1))
+    E = int(co.shape[0])
+    out = {"edges": E}
+    _l1attn_cpu.set_threads(ncores)
+    _l1attn_cpu.sparse_forward(v, q, k, coo, dmx, True)
+    t0 = time.perf_counter()
+    vo, attn = _l1attn_cpu.sparse_forward(v, q, k, coo, dmx, True)
+    _l1attn_cpu.sparse_backward(dvo, v, q, k, coo, attn, dmx, True)
+    dt = time.perf_counter() - t0
+    _l1attn_cpu.set_threads(0)
+    out["cpu_operator_package_fp32"] = {"fwd_bwd_ms": dt * 1e3, "edges_per_s": E / dt, "cores": ncores}
+    if mods is not None:
+        d = [x.double() for x in (v, q, k, dvo)]
+        t0 = time.perf_counter()
+        vo, attn = mods["l1attn_sparse_drv"].forward(d[0], d[1], d[2], coo, dmx, True)
+        mods["l1attn_sparse_drv"].backward(d[3], d[0], d[1], d[2], coo, attn, dmx, True)
+        dt = time.perf_counter() - t0
+        out["reference_fp64"] = {"fwd_bwd_ms": dt * 1e3, "edges_per_s": E / dt, "cores": 1, "kind": "reference"}
+    return out
+
+
 def cpu_baseline():
     """The reference's own CPU extension (oracle/_ref, fp64, one thread, scalar) when it was built and
     carried here, else the C restatement (oracle/liboracle.so, fp64, one thread), on a bounded sample
@@ -445,7 +477,13 @@ def cpu_baseline():
                "note": "l1attn_cpp (the CPU twin of the operators, fp32, OpenMP), same sample"}
     except Exception as e:
         log("CPU operator package not timed:", repr(e))
+    sparse = None
+    try:
+        sparse = cpu_baseline_sparse(mods, ncores)
+    except Exception as e:  # noqa: BLE001
+        log("sparse CPU baseline not timed:", repr(e))
     return {
+        "sparse_config4": sparse,
         "cpu_operator_package_fp32": pkg,
         "value": 6 * N / dt / 1e9, "unit": "GOP/s", "cores": 1, "kind": kind,
         "sample": "dense fwd+bwd fp64, B=1 T=1024 H=16 W=64 (1/128 of the headline pair-elements), %.1f s" % dt,

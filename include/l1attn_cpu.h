@@ -67,13 +67,16 @@ int l1attn_cpu_expand_coo(const void* co, int co_bits, int64_t co_stride, int64_
  * Replaces l1attn_sparse_drv.forward(v,q,k,coo,dst_mxlen,use_softmax) -> [vo, attn]
  * (cpp/l1attn_sparse_drv.cpp:13-91).  coo int32 [E, coo_stride>=3].  v, vo [B,T,H,Wv]: Wv may differ from W
  * (the reference's CUDA kernels allow it, cuda/l1attn_sparse_cuda_kernel.cu:385; its CPU loop does not).
+ * attn_zeroed != 0: the caller hands over attn holding zeros (e.g. calloc'ed) and only the slots of the edges are
+ * written; on a skewed graph the padded tensor is mostly empty slots (2 GB at 65536 tokens, dst_mxlen 2049, 4
+ * heads) and clearing it would dominate the call.  attn_zeroed == 0: every slot is written.
  */
 int l1attn_cpu_sparse_fwd_f32(const float* v, const float* q, const float* k, const int32_t* coo, int64_t coo_stride,
                               float* vo, float* attn, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv,
-                              int64_t E, int64_t dst_mxlen, int use_softmax);
+                              int64_t E, int64_t dst_mxlen, int use_softmax, int attn_zeroed);
 int l1attn_cpu_sparse_fwd_f64(const double* v, const double* q, const double* k, const int32_t* coo, int64_t coo_stride,
                               double* vo, double* attn, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv,
-                              int64_t E, int64_t dst_mxlen, int use_softmax);
+                              int64_t E, int64_t dst_mxlen, int use_softmax, int attn_zeroed);
 
 /*
  * Sparse backward -> dv, dq, dk.  Replaces l1attn_sparse_drv.backward(dvo,v,q,k,coo,attn,dst_mxlen,use_softmax)
@@ -96,10 +99,11 @@ int l1attn_cpu_sparse_bwd_f64(const double* dvo, const double* v, const double* 
  */
 int l1attn_cpu_sparse_bidi_fwd_f32(const float* vf, const float* vb, const float* q, const float* k, const int32_t* coo,
                                    int64_t coo_stride, float* vo, float* attn, int64_t B, int64_t T, int64_t H, int64_t W,
-                                   int64_t Wv, int64_t E, int64_t dst_mxlen, int use_softmax);
+                                   int64_t Wv, int64_t E, int64_t dst_mxlen, int use_softmax, int attn_zeroed);
 int l1attn_cpu_sparse_bidi_fwd_f64(const double* vf, const double* vb, const double* q, const double* k,
                                    const int32_t* coo, int64_t coo_stride, double* vo, double* attn, int64_t B, int64_t T,
-                                   int64_t H, int64_t W, int64_t Wv, int64_t E, int64_t dst_mxlen, int use_softmax);
+                                   int64_t H, int64_t W, int64_t Wv, int64_t E, int64_t dst_mxlen, int use_softmax,
+                                   int attn_zeroed);
 int l1attn_cpu_sparse_bidi_bwd_f32(const float* dvo, const float* vf, const float* vb, const float* q, const float* k,
                                    const int32_t* coo, int64_t coo_stride, const float* attn, float* dvf, float* dvb,
                                    float* dq, float* dk, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,

@@ -43,6 +43,8 @@ def lib():
                 f.restype = _c_i
                 # tensors, coo + its stride, more tensors, B T H W Wv E dst_mxlen, use_softmax
                 f.argtypes = [_c_p] * npre + [_c_i64] + [_c_p] * npost + [_c_i64] * 7 + [_c_i]
+                if name.endswith("_fwd"):
+                    f.argtypes = f.argtypes + [_c_i]  # attn_zeroed
         _lib = L
     return _lib
 
@@ -137,6 +139,13 @@ def _sparse_shapes(v, q, k, coo):
     return B, T, H, W, v.shape[3], coo.shape[0]
 
 
+def _zero_pages(shape, dtype):
+    """A zero tensor whose pages the allocator has not touched yet (numpy's zeros is calloc): the padded
+    edge-weight tensor is mostly empty slots on skewed graphs, and the library writes the slots of edges only."""
+    import numpy as np
+    return torch.from_numpy(np.zeros(shape, dtype=np.float32 if dtype == torch.float32 else np.float64))
+
+
 def _same_as(x, like, name, like_name):
     if x.shape != like.shape or x.dtype != like.dtype:
         raise RuntimeError("%s must have the shape and dtype of %s" % (name, like_name))
@@ -151,9 +160,9 @@ def sparse_forward(v, q, k, coo, dst_mxlen, use_softmax):
     M = int(dst_mxlen)
     sfx = _sfx(q)
     vo = torch.empty_like(v)
-    attn = torch.empty((B, T, M, H), dtype=q.dtype)
+    attn = _zero_pages((B, T, M, H), q.dtype)
     _check(getattr(lib(), "l1attn_cpu_sparse_fwd_" + sfx)(
-        _p(v), _p(q), _p(k), _p(coo), coo.shape[1], _p(vo), _p(attn), B, T, H, W, Wv, E, M, int(bool(use_softmax))),
+        _p(v), _p(q), _p(k), _p(coo), coo.shape[1], _p(vo), _p(attn), B, T, H, W, Wv, E, M, int(bool(use_softmax)), 1),
         "l1attn_cpu_sparse_fwd_" + sfx)
     return [vo, attn]
 
@@ -185,10 +194,10 @@ def bidi_forward(vf, vb, q, k, coo, dst_mxlen, use_softmax):
     M = int(dst_mxlen)
     sfx = _sfx(q)
     vo = torch.empty_like(vf)
-    attn = torch.empty((B, T, M, H), dtype=q.dtype)
+    attn = _zero_pages((B, T, M, H), q.dtype)
     _check(getattr(lib(), "l1attn_cpu_sparse_bidi_fwd_" + sfx)(
         _p(vf), _p(vb), _p(q), _p(k), _p(coo), coo.shape[1], _p(vo), _p(attn), B, T, H, W, Wv, E, M,
-        int(bool(use_softmax))), "l1attn_cpu_sparse_bidi_fwd_" + sfx)
+        int(bool(use_softmax)), 1), "l1attn_cpu_sparse_bidi_fwd_" + sfx)
     return [vo, attn]
 
 

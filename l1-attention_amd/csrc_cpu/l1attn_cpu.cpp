@@ -133,24 +133,27 @@ int l1attn_cpu_expand_coo(const void* co, int co_bits, int64_t co_stride, int64_
 
 #define L1CPU_SPARSE(SFX, F)                                                                                                 \
 	int l1attn_cpu_sparse_fwd_##SFX(const F* v, const F* q, const F* k, const int32_t* coo, int64_t cs, F* vo, F* attn,      \
-	                                int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E, int64_t M, int sm)    \
+	                                int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E, int64_t M, int sm,    \
+	                                int attn_zeroed)                                                                         \
 	{                                                                                                                        \
 		if (bad_dims(B, T, H, W) || Wv < 1) return L1ATTN_CPU_ERR_ARG;                                                       \
 		if (int rc = check_coo(coo, cs, E, T, M)) return rc;                                                                 \
 		if (B * T * H == 0) return 0;                                                                                        \
 		if (!v || !q || !k || !vo || (M > 0 && !attn)) return L1ATTN_CPU_ERR_ARG;                                            \
-		table().sparse_fwd_##SFX(v, nullptr, q, k, coo, cs, vo, attn, B, T, H, W, Wv, E, M, sm != 0, threads());             \
+		table().sparse_fwd_##SFX(v, nullptr, q, k, coo, cs, vo, attn, B, T, H, W, Wv, E, M, sm != 0, attn_zeroed != 0,       \
+		                         threads());                                                                                 \
 		return 0;                                                                                                            \
 	}                                                                                                                        \
 	int l1attn_cpu_sparse_bidi_fwd_##SFX(const F* vf, const F* vb, const F* q, const F* k, const int32_t* coo, int64_t cs,   \
 	                                     F* vo, F* attn, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, int64_t E,  \
-	                                     int64_t M, int sm)                                                                  \
+	                                     int64_t M, int sm, int attn_zeroed)                                                 \
 	{                                                                                                                        \
 		if (bad_dims(B, T, H, W) || Wv < 1) return L1ATTN_CPU_ERR_ARG;                                                       \
 		if (int rc = check_coo(coo, cs, E, T, M)) return rc;                                                                 \
 		if (B * T * H == 0) return 0;                                                                                        \
 		if (!vf || !vb || !q || !k || !vo || (M > 0 && !attn)) return L1ATTN_CPU_ERR_ARG;                                    \
-		table().bidi_fwd_##SFX(vf, vb, q, k, coo, cs, vo, attn, B, T, H, W, Wv, E, M, sm != 0, threads());                   \
+		table().bidi_fwd_##SFX(vf, vb, q, k, coo, cs, vo, attn, B, T, H, W, Wv, E, M, sm != 0, attn_zeroed != 0,             \
+		                       threads());                                                                                   \
 		return 0;                                                                                                            \
 	}                                                                                                                        \
 	int l1attn_cpu_sparse_bwd_##SFX(const F* dvo, const F* v, const F* q, const F* k, const int32_t* coo, int64_t cs,        \

@@ -11,13 +11,13 @@ struct L1CpuTable {
 	void (*dense_bwd_f64)(const double*, const double*, const double*, double*, double*, int64_t, int64_t, int64_t, int64_t,
 	                      int);
 	void (*sparse_fwd_f32)(const float*, const float*, const float*, const float*, const int32_t*, int64_t, float*, float*,
-	                       int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, int);
+	                       int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, bool, int);
 	void (*sparse_fwd_f64)(const double*, const double*, const double*, const double*, const int32_t*, int64_t, double*,
-	                       double*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, int);
+	                       double*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, bool, int);
 	void (*bidi_fwd_f32)(const float*, const float*, const float*, const float*, const int32_t*, int64_t, float*, float*,
-	                     int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, int);
+	                     int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, bool, int);
 	void (*bidi_fwd_f64)(const double*, const double*, const double*, const double*, const int32_t*, int64_t, double*,
-	                     double*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, int);
+	                     double*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, bool, int);
 	void (*sparse_bwd_f32)(const float*, const float*, const float*, const float*, const float*, const int32_t*, int64_t,
 	                       const float*, float*, float*, float*, float*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,
 	                       int64_t, bool, int);
