@@ -126,7 +126,7 @@ def check_scalar_prefetch(asm_text, kernels=None):
     return n_loads
 
 
-_ASM_STMT = re.compile(r"\basm\s*(?:volatile\s*)?\(")
+_ASM_STMT = re.compile(r"(?:\b|__)asm(?:__)?\s*(?:(?:volatile|__volatile__|goto)\s*)*\(")  # asm, __asm__, __asm
 SCALAR_LOAD_HELPER = ("sload.h", "sload32")  # the one function whose inline asm may issue scalar loads
 
 

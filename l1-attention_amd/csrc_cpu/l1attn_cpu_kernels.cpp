@@ -137,7 +137,7 @@ void sparse_fwd(const F* v, const F* vb, const F* q, const F* k, const int32_t* 
 			F* slots = attn + (b * T + d) * M * H;
 			// the padded tensor is mostly empty slots on skewed graphs: a caller that hands over zeroed memory
 			// (calloc: pages that were never touched) saves touching all of it
-			if (!attn_zeroed) std::memset(slots, 0, sizeof(F) * M * H);
+			if (!attn_zeroed && M > 0) std::memset(slots, 0, sizeof(F) * M * H);
 			F* out = vo + (b * T + d) * vrow;
 			std::memset(out, 0, sizeof(F) * vrow);
 			const F* qd = q + (b * T + d) * row;

@@ -253,6 +253,8 @@ _Z5kern2v: ; @k
         build.check_asm_sources({"sload.h": ok["sload.h"].replace("sload32", "other")})
     with pytest.raises(RuntimeError, match="issues buffer_load_dword"):
         build.check_asm_sources({"dense.hip": 'void f()\n{\n\tasm volatile("v_nop\\n\\tbuffer_load_dword %0, %1, %2, 0 offen" : "=v"(x) : "v"(o), "s"(r));\n}\n'})
+    with pytest.raises(RuntimeError, match="issues global_load_dword"):
+        build.check_asm_sources({"coo.hip": 'void f()\n{\n\t__asm__ __volatile__("global_load_dword %0, %1, off" : "=v"(x) : "v"(a));\n}\n'})
     with pytest.raises(RuntimeError, match="issues ds_read_b32"):
         build.check_asm_sources({"fused.hip": 'void f()\n{\n\tasm("ds_read_b32 %0, %1" : "=v"(x) : "v"(o));\n}\n'})
 
