@@ -73,3 +73,38 @@ def bidi_powerlaw_graph(bi_mod, dev, B, T, H, W, seed=1005):
     rvo = cf.bidi_value(*ref_leaves, coo, True)
     ref = (rvo.detach(),) + torch.autograd.grad(rvo, ref_leaves, dvo.double())
     return co.shape[0], dmx, [cf.rel_err(x, y) for x, y in zip(got, ref)]
+
+
+def dense_sampled_rows(drv, dev, B, T, H, W, layernorm, rows, seed=1003):
+    """Third baseline configuration at a size where no full float64 yardstick fits: sampled (batch, row) pairs of
+    the logits, dq and dk against the defining sums in float64, the checksum sum_t dq = -sum_s dk over everything,
+    and bitwise repeatability of the backward.  `drv` is a driver binding with dense_forward(q, k) -> [attn] and
+    dense_backward(d_attn, q, k) -> [dq, dk] (the reference's native interface, cuda/l1attn_cuda_drv.cpp:106-109).
+    layernorm: inputs scaled to zero mean and unit variance per token and head, the configuration's second input set.
+    Returns the worst errors (logits, dq, dk, checksum relative to the largest column sum)."""
+    import math
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q = torch.randn(B, T, H, W, generator=g, device=dev)
+    k = torch.randn(B, T, H, W, generator=g, device=dev)
+    if layernorm:
+        q = torch.nn.functional.layer_norm(q, (W,))
+        k = torch.nn.functional.layer_norm(k, (W,))
+    da = torch.empty(B, T, T, H, device=dev)
+    for b in range(B):  # one batch at a time: 1 GiB each at the full size
+        da[b].normal_(generator=g)
+    a = drv.dense_forward(q, k)[0]
+    dq, dk = drv.dense_backward(da, q, k)
+    dq2, dk2 = drv.dense_backward(da, q, k)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2)
+    scale = -1.0 / math.sqrt(W)
+    worst = [0.0, 0.0, 0.0]
+    for b, r in rows:
+        diff = q[b, r].double()[None] - k[b].double()                      # [S,H,W]: row r as dst token
+        ra = scale * diff.abs().sum(-1)
+        rdq = scale * (torch.sign(diff) * da[b, :, r, :, None].double()).sum(0)
+        diff = q[b].double() - k[b, r].double()[None]                      # [T,H,W]: row r as src token
+        rdk = -scale * (torch.sign(diff) * da[b, r, :, :, None].double()).sum(0)
+        errs = (cf.rel_err(a[b, :, r, :], ra), cf.rel_err(dq[b, r], rdq), cf.rel_err(dk[b, r], rdk))
+        worst = [max(x, y) for x, y in zip(worst, errs)]
+    sq, sk = dq.double().sum(1), dk.double().sum(1)
+    return worst + [float((sq + sk).abs().max()) / float(sq.abs().max())]

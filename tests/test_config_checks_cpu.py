@@ -23,3 +23,11 @@ def test_bidi_powerlaw_graph_on_the_cpu_package():
     E, dmx, errs = cc.bidi_powerlaw_graph(l1attn_sparse_bidi_cpp, torch.device("cpu"), 1, 2048, 2, 64)
     assert E > 2 * 2048 and dmx > 128            # long segments are part of the case
     assert errs[0] <= cc.FWD_TOL and max(errs[1:]) <= cc.BWD_TOL
+
+
+def test_dense_sampled_rows_on_the_cpu_package():
+    import _l1attn_cpu
+    for layernorm in (False, True):
+        errs = cc.dense_sampled_rows(_l1attn_cpu, torch.device("cpu"), 2, 160, 4, 32, layernorm,
+                                     [(0, 0), (1, 159), (1, 77)])
+        assert errs[0] <= cc.FWD_TOL and errs[1] <= cc.BWD_TOL and errs[2] <= cc.BWD_TOL and errs[3] <= 1e-4

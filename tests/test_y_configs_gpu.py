@@ -31,6 +31,18 @@ def test_config2_full_batch_with_downstream_softmax_and_einsum():
     assert errs[0] <= cc.FWD_TOL and errs[1] <= cc.FWD_TOL and errs[2] <= cc.BWD_TOL and errs[3] <= cc.BWD_TOL
 
 
+def test_config3_full_size_layernorm_scaled_inputs():
+    """B=8, T=4096, H=16, W=64 with the configuration's second input set (unit variance per token and head):
+    sampled rows of the logits and both gradients in float64, the checksum and bitwise repeatability.  (The N(0,1)
+    input set at this size is tests/test_dense_gpu.py::test_dense_headline_size_properties.)"""
+    print("case config 3 at full size, LayerNorm-scaled inputs", flush=True)
+    import _l1attn_hip as drv
+    errs = cc.dense_sampled_rows(drv, DEV, 8, 4096, 16, 64, True, [(0, 0), (3, 5), (7, 4095), (5, 2049)])
+    print("errors (logits, dq, dk, checksum):", errs, flush=True)
+    assert errs[0] <= cc.FWD_TOL and errs[1] <= cc.BWD_TOL and errs[2] <= cc.BWD_TOL and errs[3] <= 1e-4
+    torch.cuda.empty_cache()
+
+
 def test_config4_full_size():
     """B=4, T=4096, H=8, W=32, degrees U{1..64}: about 133 k edges."""
     print("case config 4 at full size", flush=True)
