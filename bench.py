@@ -295,6 +295,18 @@ def extra_legs():
         del q, k, a32, afx
         torch.cuda.empty_cache()
     res["instruction_rates"] = instruction_rates()
+    # column ranks of the long-sequence backward: library block radix sort against the merge sort of rank_sort.hip
+    B, T, H, W = 8, 4096, 16, 64
+    q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
+    q, k = q.to(dev), k.to(dev)
+    rq, rk = torch.empty_like(q), torch.empty_like(k)
+    L, st = drv.lib(), drv.stream_of(q)
+    res["column_ranks_B8_T4096_H16_W64"] = {
+        "library_radix_sort_ms": time_gpu(lambda: L.l1attn_dense_column_ranks_f32(
+            drv.ptr(q), drv.ptr(k), drv.ptr(rq), drv.ptr(rk), B, T, H, W, st), 10),
+        "merge_sort_ms": time_gpu(lambda: L.l1attn_dense_column_ranks_merge_f32(
+            drv.ptr(q), drv.ptr(k), drv.ptr(rq), drv.ptr(rk), B, T, H, W, st), 10)}
+    log(json.dumps(res["column_ranks_B8_T4096_H16_W64"]))
     return res
 
 

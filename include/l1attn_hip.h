@@ -113,6 +113,14 @@ int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k,
  */
 int l1attn_dense_column_ranks_f32(const float* q, const float* k, float* rq, float* rk,
                                   int64_t B, int64_t T, int64_t H, int64_t W, void* stream);
+/*
+ * The same ranks (identical rq, rk) from a merge sort written for this library instead of the library block
+ * radix sort behind l1attn_dense_column_ranks_f32.  l1attn_dense_bwd_f32 uses it only when the environment
+ * holds L1ATTN_RANK_SORT=merge (read once per process); kept beside the other until both have been timed on a
+ * GPU.  No counterpart in the reference.
+ */
+int l1attn_dense_column_ranks_merge_f32(const float* q, const float* k, float* rq, float* rk,
+                                        int64_t B, int64_t T, int64_t H, int64_t W, void* stream);
 
 /*
  * Experimental: the f32 forward on fixed point.  q and k of every (batch, head) are converted once to

@@ -97,6 +97,8 @@ def lib():
             f.argtypes = [_c_p] * 8 + [_c_i64] * 5 + [_c_p]
         L.l1attn_dense_column_ranks_f32.restype = _c_i
         L.l1attn_dense_column_ranks_f32.argtypes = [_c_p] * 4 + [_c_i64] * 4 + [_c_p]
+        L.l1attn_dense_column_ranks_merge_f32.restype = _c_i
+        L.l1attn_dense_column_ranks_merge_f32.argtypes = [_c_p] * 4 + [_c_i64] * 4 + [_c_p]
         L.l1attn_expand_coo_workspace_bytes.restype = _c_sz
         L.l1attn_expand_coo_workspace_bytes.argtypes = [_c_i64]
         L.l1attn_expand_coo.restype = _c_i

@@ -28,6 +28,7 @@
 #include "xcd.h"
 #include "fixed.h"
 #include <math.h>
+#include <stdlib.h>
 #include <algorithm>
 
 namespace {
@@ -950,6 +951,18 @@ struct BwdPlan {
 
 constexpr int N_CU = 256;
 
+// Which kernel computes the column ranks of the long-sequence backward: the library block radix sort
+// (dense_rank.hip, the default: it is the one that has run the GPU tests) or the merge sort of rank_sort.hip
+// when the environment holds L1ATTN_RANK_SORT=merge.  Both give the same ranks; the choice is read once.
+bool l1_rank_sort_is_merge()
+{
+	static const bool merge = [] {
+		const char* e = getenv("L1ATTN_RANK_SORT");
+		return e && e[0] == 'm';
+	}();
+	return merge;
+}
+
 BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 {
 	BwdPlan p{};
@@ -1220,7 +1233,8 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 		const float* qa = q + b0 * T * HW;
 		const float* ka = k + b0 * T * HW;
 		if (p.rank) {
-			const int rc = l1_launch_column_ranks(qa, ka, rq, rk, nb, T, H, W, st);
+			const int rc = l1_rank_sort_is_merge() ? l1_launch_column_ranks_merge(qa, ka, rq, rk, nb, T, H, W, st)
+			                                       : l1_launch_column_ranks(qa, ka, rq, rk, nb, T, H, W, st);
 			if (rc != L1ATTN_OK) return rc;
 			qa = rq;
 			ka = rk;

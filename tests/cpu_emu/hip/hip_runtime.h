@@ -68,6 +68,10 @@ inline void wave_sync() { wave_barrier[flat_tid() >> 6]->arrive_and_wait(); }
 using std::min;
 using std::max;
 
+#include <string.h>
+static inline unsigned __float_as_uint(float x) { unsigned u; memcpy(&u, &x, 4); return u; }
+static inline float __uint_as_float(unsigned u) { float x; memcpy(&x, &u, 4); return x; }
+
 // value of the wave's first active lane; the kernels built here only pass wave-uniform values
 static inline int __builtin_amdgcn_readfirstlane(int x) { return x; }
 // Cross-lane read within the wave: every lane of the wave must call it (uniform control flow).

@@ -233,3 +233,63 @@ def test_fixed_point_prepass_kernels_on_cpu(tmp_path):
         # half a step from rint, up to a quarter more from the fp32 rounding of the quotient below 2^23
         assert np.all(np.abs(decoded - x) <= 0.7500001 * g_ref[:, None, :, None])
     assert np.all(uq[1, :, 2] == 2 ** 31) and np.all(uk[1, :, 2] == 2 ** 31)
+
+
+def _reference_ranks(q, k):
+    """rq, rk of one [B,T,H,W] pair by their definition, with numpy: per column, rk = 2 * #{k' < k} - 1/2 and
+    rq = 2 * #{k' < q}, minus one where q ties with no k.  -0 and +0 are equal."""
+    qn, kn = q.numpy().astype(np.float64) + 0.0, k.numpy().astype(np.float64) + 0.0
+    B, T, H, W = qn.shape
+    rq, rk = np.empty_like(qn), np.empty_like(kn)
+    for b in range(B):
+        for h in range(H):
+            for w in range(W):
+                ks = np.sort(kn[b, :, h, w])
+                less_k = np.searchsorted(ks, kn[b, :, h, w], side="left")
+                rk[b, :, h, w] = 2 * less_k - 0.5
+                less_q = np.searchsorted(ks, qn[b, :, h, w], side="left")
+                tie = np.searchsorted(ks, qn[b, :, h, w], side="right") > less_q
+                rq[b, :, h, w] = 2 * less_q - np.where(tie, 0, 1)
+    return rq, rk
+
+
+@pytest.mark.parametrize("shape", [(1, 4096, 1, 2), (1, 1000, 2, 2), (2, 300, 1, 3), (1, 2049, 1, 2), (1, 5000, 1, 1),
+                                   (1, 1, 1, 5), (1, 513, 3, 1)])
+def test_merge_sort_column_ranks_on_cpu(tmp_path, shape):
+    """The merge-sort rank kernel (csrc/rank_sort.hip; registers, LDS and barriers only) under AddressSanitizer:
+    every items-per-thread instantiation (T up to 512, 1024, 2048, 4096, 8192), ragged lengths (padding keys),
+    planted ties between q and k, repeated k values, both zeros; ranks equal their definition exactly, and
+    clamp(rq - rk, 0, 1) is 1, 1/2, 0 for q >, ==, < k on every pair of a column."""
+    exe = str(tmp_path / "run_ranks")
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
+                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_ranks.cpp"), "-o", exe],
+                   check=True)
+    B, T, H, W = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))
+    if T > 8:
+        idx = torch.randperm(T, generator=g)[: T // 8]
+        q[:, idx] = k[:, idx.flip(0)]                    # ties between q and k
+        k[:, : T // 16] = k[:, T // 16: 2 * (T // 16)]   # repeated k values
+        q[0, 0, 0, 0], k[0, 1, 0, 0] = 0.0, -0.0
+    if W > 1:
+        q[..., 1] = torch.round(q[..., 1])               # a column on a coarse grid: long runs of equal keys
+        k[..., 1] = torch.round(k[..., 1])
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    with open(fin, "wb") as f:
+        f.write(struct.pack("4q", B, T, H, W))
+        f.write(q.numpy().tobytes())
+        f.write(k.numpy().tobytes())
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
+    r = subprocess.run([exe, fin, fout], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, (r.returncode, r.stderr[-2000:])
+    raw = open(fout, "rb").read()
+    n = B * T * H * W
+    rq = np.frombuffer(raw, np.float32, n).reshape(B, T, H, W)
+    rk = np.frombuffer(raw, np.float32, n, n * 4).reshape(B, T, H, W)
+    ref_rq, ref_rk = _reference_ranks(q, k)
+    assert np.array_equal(rq, ref_rq) and np.array_equal(rk, ref_rk)
+    if T <= 1000:  # all pairs of every column
+        hv = np.clip(rq[:, :, None] - rk[:, None], 0.0, 1.0)             # [B,T(dst),S(src),H,W]
+        sign = np.sign((q.numpy()[:, :, None] + 0.0) - (k.numpy()[:, None] + 0.0))
+        assert np.array_equal(2 * hv - 1, sign)
