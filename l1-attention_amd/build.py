@@ -231,6 +231,74 @@ def check_hot_kernels(res):
         raise RuntimeError("hot-path kernels must not spill:\n" + "\n".join(problems))
 
 
+def loop_profiles(asm_text, kernel_substr):
+    """Instruction mix of every loop (a branch back to an earlier label) of the kernels whose mangled name contains
+    kernel_substr: [{"kernel", "first", "last", "valu", "salu", "smem", "lds", "vmem", "waitcnt", "other"}]."""
+    out = []
+    lines = asm_text.split("\n")
+    i = 0
+    while i < len(lines):
+        l = lines[i]
+        if l.startswith("_Z") and kernel_substr in l and ":" in l.split(";")[0]:
+            name = l.split(":")[0]
+            ins, labels = [], {}
+            i += 1
+            while i < len(lines) and not lines[i].strip().startswith(".Lfunc_end"):
+                t = lines[i].split(";")[0].strip()
+                i += 1
+                m = re.match(r"^(\.LBB\d+_\d+):", t)
+                if m:
+                    labels[m.group(1)] = len(ins)
+                elif t and t[0] not in ".;" and not t.endswith(":"):
+                    ins.append(t)
+            for n, t in enumerate(ins):
+                m = re.search(r"s_c?branch\w* (\.LBB\d+_\d+)", t)
+                if m and labels.get(m.group(1), n + 1) <= n:
+                    mix = dict(kernel=name, first=labels[m.group(1)], last=n, valu=0, salu=0, smem=0, lds=0, vmem=0,
+                               waitcnt=0, other=0)
+                    for u in ins[labels[m.group(1)]:n + 1]:
+                        op = u.split()[0]
+                        kind = ("valu" if op.startswith("v_") else "waitcnt" if op.startswith("s_waitcnt") else
+                                "smem" if op.startswith(("s_load", "s_buffer_load")) else "salu" if op.startswith("s_") else
+                                "lds" if op.startswith("ds_") else
+                                "vmem" if op.startswith(("buffer_", "global_", "flat_", "scratch_")) else "other")
+                        mix[kind] += 1
+                    out.append(mix)
+        else:
+            i += 1
+    return out
+
+
+# The loops that carry the headline path: kernel, pair-elements a lane finishes per iteration, vector-ALU
+# instructions the kernel's formulation needs per pair-element, and the most the build accepts (what is above the
+# formulation's own count is loop overhead the compiler adds: address arithmetic, staging, the flush).
+HOT_LOOPS = (
+    ("dense_fwd_f32_pipeILi64ELb0E", 8 * 64, 2, 2.30),                    # eight src rows of 64 columns per lane
+    ("dense_fwd_f32_pipeILi32ELb0E", 8 * 32, 2, 2.55),
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E", 4 * 64, 3, 3.20),  # four src rows against 64 dst tokens, ranks
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1E", 4 * 64, 4, 4.25),  # the same with the sign from the difference
+)
+
+
+def check_hot_loops(asm_text, table=HOT_LOOPS):
+    """Vector-ALU instructions per pair-element in the loops of the headline kernels, from the listing: the loop taken
+    for a kernel is the smallest one that holds at least the algorithm's own instructions.  A compiler that starts
+    to spend more than the accepted overhead there fails the build instead of showing up as a slower benchmark.
+    Returns {kernel substring: instructions per pair-element}."""
+    found = {}
+    for sub, pairs, own, most in table:
+        need = pairs * own
+        loops = [p for p in loop_profiles(asm_text, sub) if p["valu"] >= need]
+        if not loops:
+            raise RuntimeError("hot-loop check: no loop of %s holds %d vector instructions" % (sub, need))
+        per = min(p["valu"] for p in loops) / float(pairs)
+        if per > most:
+            raise RuntimeError("hot-loop check: %s spends %.2f vector instructions per pair-element (accepted: %.2f)"
+                               % (sub, per, most))
+        found[sub] = per
+    return found
+
+
 def build(verbose=False):
     sys.path.insert(0, HERE)
     try:
@@ -291,6 +359,9 @@ def build(verbose=False):
         print("scalar-prefetch check: %d loads verified" % n)
     res = kernel_resources(asm)
     check_hot_kernels(res)
+    per_pair = check_hot_loops(asm)
+    if verbose:
+        print("vector instructions per pair-element:", per_pair)
     with open(os.path.join(HERE, "build", "dense_kernel_resources.txt"), "w") as f:
         for name in sorted(res):
             f.write("%s %s\n" % (name, " ".join("%s=%d" % kv for kv in sorted(res[name].items()))))

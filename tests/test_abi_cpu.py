@@ -529,3 +529,31 @@ def test_native_module_stand_ins_without_a_gpu(monkeypatch):
     vo, attn = l1attn_sparse_bidi_cuda_drv.forward(v, vb, q, k, coo, 3, False)
     grads = l1attn_sparse_bidi_cuda_drv.backward(torch.zeros_like(vo), v, vb, q, k, coo, attn, dmx.item(), False)
     assert len(grads) == 4 and all(g.shape == v.shape for g in grads)
+
+
+def test_build_checks_the_instruction_density_of_the_hot_loops():
+    """build.py counts the vector-ALU instructions of the headline kernels' loops on the listing and fails when a
+    loop spends more per pair-element than accepted (the algorithm itself: 2 forward, 3 backward)."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import build
+    body = "\n".join(["\tv_subrev_f32_e32 v1, s4, v2", "\tv_add_f32_e64 v3, v3, |v1|"] * 8)
+    listing = """
+_Z4kernv: ; @k
+	s_load_dwordx2 s[0:1], s[4:5], 0x0
+.LBB0_1: ; %loop
+""" + body + """
+	s_add_u32 s2, s2, 1
+	s_waitcnt lgkmcnt(0)
+	ds_read_b32 v9, v8
+	s_cbranch_scc1 .LBB0_1
+	s_endpgm
+.Lfunc_end0:
+"""
+    (loop,) = build.loop_profiles(listing, "kern")
+    assert (loop["valu"], loop["salu"], loop["waitcnt"], loop["lds"], loop["smem"]) == (16, 2, 1, 1, 0)
+    assert build.check_hot_loops(listing, (("kernv", 8, 2, 2.0),)) == {"kernv": 2.0}
+    with pytest.raises(RuntimeError, match="2.00 vector instructions per pair-element"):
+        build.check_hot_loops(listing, (("kernv", 8, 2, 1.9),))
+    with pytest.raises(RuntimeError, match="no loop"):
+        build.check_hot_loops(listing, (("kernv", 16, 2, 4.0),))
