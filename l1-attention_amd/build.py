@@ -127,13 +127,13 @@ def check_scalar_prefetch(asm_text, kernels=None):
 
 
 _ASM_STMT = re.compile(r"(?:\b|__)asm(?:__)?\s*(?:(?:volatile|__volatile__|goto)\s*)*\(")  # asm, __asm__, __asm
-SCALAR_LOAD_HELPER = ("sload.h", "sload32")  # the one function whose inline asm may issue scalar loads
+SCALAR_LOAD_HELPER = ("sload.h", "sload32")  # the one header, and the name its loading helpers start with
 
 
 def check_asm_sources(files=None):
     """Source-level twin of check_inline_asm_loads, so that the rule also covers templates nobody instantiates
     yet: no `asm` statement under csrc/ may contain a vector-memory, LDS or returning-atomic load, and `s_load`
-    may appear only in the body of the one helper named above.  `files`: {name: text}, default csrc/*."""
+    may appear only in the helpers of the one header named above.  `files`: {name: text}, default csrc/*."""
     if files is None:
         files = {}
         for path in sorted(glob.glob(os.path.join(HERE, "csrc", "*"))):
@@ -142,6 +142,9 @@ def check_asm_sources(files=None):
                     files[os.path.basename(path)] = f.read()
     problems = []
     for name, text in sorted(files.items()):
+        # comments out (line breaks kept for the line numbers): prose must not look like code to the scan below
+        text = re.sub(r"/\*.*?\*/", lambda c: "\n" * c.group(0).count("\n"), text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
         for m in _ASM_STMT.finditer(text):
             depth, i = 1, m.end()
             while i < len(text) and depth:  # the statement up to its closing parenthesis
@@ -156,7 +159,7 @@ def check_asm_sources(files=None):
                 elif op.startswith("s_load_") or op.startswith("s_buffer_load"):
                     # the enclosing function: the last definition header before the statement
                     heads = re.findall(r"\b(\w+)\s*\([^;{}]*\)\s*\{", text[:m.start()])
-                    if (name, heads[-1] if heads else "") != SCALAR_LOAD_HELPER:
+                    if name != SCALAR_LOAD_HELPER[0] or not (heads and heads[-1].startswith(SCALAR_LOAD_HELPER[1])):
                         problems.append("%s:%d: %s outside %s()" % (name, line, op, SCALAR_LOAD_HELPER[1]))
     if problems:
         raise RuntimeError("inline asm may not issue loads the compiler does not track:\n" + "\n".join(problems))

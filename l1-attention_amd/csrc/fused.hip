@@ -86,6 +86,10 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restric
 		}
 #pragma unroll
 		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+		// take the q row here: left alone, the compiler waits for each of its loads at the first use, inside the
+		// src loop, where the sixteen waits are then issued once per src token
+#pragma unroll
+		for (int w = 0; w < W; w++) asm volatile("" : "+v"(qr[w]));
 	}
 	float den = 0.0f;
 	const int64_t row = (int64_t)H * W;
@@ -119,6 +123,47 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restric
 // next chunk issued before the VALU work on the current one.  A row holds an even number of chunks (2*W/32), so a
 // chunk's buffer is fixed by its place in the row.  The load issued after a row's last chunk is the first k chunk
 // of the next row, clamped to the last row at the end (read, never used), and drained after the loop.
+
+// Chunk C of a src token's 2*W/32 (k chunks first, then v chunks), then the chunks after it.
+template <int W, int C>
+__device__ __forceinline__ void fused_pipe_chunks(const float (&qr)[W], float (&acc)[W], float& a, float& p, float& den,
+                                                  float scale, f32x16& b0l, f32x16& b0h, f32x16& b1l, f32x16& b1h,
+                                                  const float* krow, const float* vrow, const float* knext)
+{
+	constexpr int CPR = W / 32;  // chunks per k row and per v row
+	f32x16& lo = (C & 1) == 0 ? b0l : b1l;  // this chunk's buffer
+	f32x16& hi = (C & 1) == 0 ? b0h : b1h;
+	f32x16& nl = (C & 1) == 0 ? b1l : b0l;  // the next chunk's
+	f32x16& nh = (C & 1) == 0 ? b1h : b0h;
+	// (the scheduler may not move the previous chunk's VALU work below this chunk's wait: the wait would then
+	// come a few instructions after the load it waits for)
+	__builtin_amdgcn_sched_barrier(0);
+	swait32(lo, hi);
+	__builtin_amdgcn_sched_barrier(0);
+	// the chunk after this one: the rest of the k row, then the v row, then the next token's k row
+	if constexpr (C + 1 < CPR) sload32_at<(C + 1) * 128>(nl, nh, krow);
+	else if constexpr (C + 1 < 2 * CPR) sload32_at<(C + 1 - CPR) * 128>(nl, nh, vrow);
+	else sload32(nl, nh, knext);
+	__builtin_amdgcn_sched_barrier(0);
+	if constexpr (C < CPR) {
+#pragma unroll
+		for (int i = 0; i < 16; i++) a += fabsf(qr[C * 32 + i] - lo[i]);
+#pragma unroll
+		for (int i = 0; i < 16; i++) a += fabsf(qr[C * 32 + 16 + i] - hi[i]);
+	} else {
+		if constexpr (C == CPR) {
+			p = expf(a * scale);
+			den += p;
+		}
+#pragma unroll
+		for (int i = 0; i < 16; i++) acc[(C - CPR) * 32 + i] += p * lo[i];
+#pragma unroll
+		for (int i = 0; i < 16; i++) acc[(C - CPR) * 32 + 16 + i] += p * hi[i];
+	}
+	if constexpr (C + 1 < 2 * CPR)
+		fused_pipe_chunks<W, C + 1>(qr, acc, a, p, den, scale, b0l, b0h, b1l, b1h, krow, vrow, knext);
+}
+
 template <int W>
 __global__ __launch_bounds__(256) void fused_fwd_f32_pipe(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ vo,
@@ -146,9 +191,12 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_pipe(const float* __restric
 		}
 #pragma unroll
 		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+		// take the q row here: left alone, the compiler waits for each of its loads at the first use, inside the
+		// src loop, where the sixteen waits are then issued once per src token
+#pragma unroll
+		for (int w = 0; w < W; w++) asm volatile("" : "+v"(qr[w]));
 	}
 	float den = 0.0f;
-	constexpr int CPR = W / 32;  // chunks per k row and per v row
 	const int64_t row = (int64_t)H * W;
 	const float* const kb = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;  // src token 0 of this (b,h): wave-uniform
 	const float* const vb = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
@@ -157,46 +205,9 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_pipe(const float* __restric
 	__builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
 	for (int s = 0; s < Tn; s++) {
-		const float* const krow = kb + s * row;
-		const float* const vrow = vb + s * row;
-		const float* const knext = kb + min(s + 1, Tn - 1) * row;
 		float a = 0.0f, p = 0.0f;
-#pragma unroll
-		for (int c = 0; c < 2 * CPR; c++) {
-			// the chunk after this one: the rest of the k row, then the v row, then the next token's k row
-			const float* const nxt = c + 1 < CPR ? krow + (c + 1) * 32 : c + 1 < 2 * CPR ? vrow + (c + 1 - CPR) * 32 : knext;
-			// (the scheduler may not move the previous chunk's VALU work below this chunk's wait: the wait would
-			// then come a few instructions after the load it waits for)
-			__builtin_amdgcn_sched_barrier(0);
-			if ((c & 1) == 0) {
-				swait32(b0l, b0h);
-				__builtin_amdgcn_sched_barrier(0);
-				sload32(b1l, b1h, nxt);
-				__builtin_amdgcn_sched_barrier(0);
-			} else {
-				swait32(b1l, b1h);
-				__builtin_amdgcn_sched_barrier(0);
-				sload32(b0l, b0h, nxt);
-				__builtin_amdgcn_sched_barrier(0);
-			}
-			const f32x16& lo = (c & 1) == 0 ? b0l : b1l;
-			const f32x16& hi = (c & 1) == 0 ? b0h : b1h;
-			if (c < CPR) {
-#pragma unroll
-				for (int i = 0; i < 16; i++) a += fabsf(qr[c * 32 + i] - lo[i]);
-#pragma unroll
-				for (int i = 0; i < 16; i++) a += fabsf(qr[c * 32 + 16 + i] - hi[i]);
-			} else {
-				if (c == CPR) {
-					p = expf(a * scale);
-					den += p;
-				}
-#pragma unroll
-				for (int i = 0; i < 16; i++) acc[(c - CPR) * 32 + i] += p * lo[i];
-#pragma unroll
-				for (int i = 0; i < 16; i++) acc[(c - CPR) * 32 + 16 + i] += p * hi[i];
-			}
-		}
+		fused_pipe_chunks<W, 0>(qr, acc, a, p, den, scale, b0l, b0h, b1l, b1h, kb + s * row, vb + s * row,
+		                        kb + min(s + 1, Tn - 1) * row);
 	}
 	swait32(b0l, b0h);  // drain the last prefetch before the wave ends
 	if (store) {

@@ -20,6 +20,15 @@ __device__ __forceinline__ void sload32(f32x16& lo, f32x16& hi, const float* p)
 	// early-clobber outputs: the second load must still see the pointer
 	asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40" : "=&s"(lo), "=&s"(hi) : "s"(p));
 }
+// The same load from p + BYTES (a compile-time offset inside the row: no scalar add, no second pointer).
+template <int BYTES>
+__device__ __forceinline__ void sload32_at(f32x16& lo, f32x16& hi, const float* p)
+{
+	static_assert(BYTES >= 0 && BYTES % 4 == 0 && BYTES + 0x40 < (1 << 20), "immediate offset of a scalar load");
+	asm volatile("s_load_dwordx16 %0, %2, %3\n\ts_load_dwordx16 %1, %2, %4"
+	             : "=&s"(lo), "=&s"(hi)
+	             : "s"(p), "n"(BYTES), "n"(BYTES + 0x40));
+}
 __device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
 {
 	asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(lo), "+s"(hi));

@@ -31,6 +31,11 @@ static inline void sload32(f32x16& lo, f32x16& hi, const float* p)
 	emu_sload::pending.push_back({&lo, &hi, p});
 	emu_sload::outstanding++;
 }
+template <int BYTES>
+static inline void sload32_at(f32x16& lo, f32x16& hi, const float* p)
+{
+	sload32(lo, hi, p + BYTES / 4);
+}
 static inline void swait32(f32x16&, f32x16&)
 {
 	for (const auto& x : emu_sload::pending) {
