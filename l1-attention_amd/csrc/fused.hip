@@ -373,6 +373,9 @@ __global__ __launch_bounds__(256) void fused_bwd_dv_tile(const float* __restrict
 		}
 #pragma unroll
 		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+		// take the k row here rather than at its first use inside the dst loop (see fused_fwd_f32_tile)
+#pragma unroll
+		for (int w = 0; w < W; w++) asm volatile("" : "+v"(kr[w]));
 	}
 	const int64_t row = (int64_t)H * W;
 	const float* qp = q + (((int64_t)b * Tn) * H + h) * (int64_t)W;    // dst token 0 of this (b,h): wave-uniform
