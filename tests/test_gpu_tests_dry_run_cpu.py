@@ -27,6 +27,7 @@ def gpu_tests_on_cpu(monkeypatch):
 def test_stand_in_and_model_block_tests_walk_on_the_cpu_package(gpu_tests_on_cpu):
     gpu_tests_on_cpu.test_native_module_stand_ins_on_the_gpu()
     gpu_tests_on_cpu.test_model_blocks_on_the_gpu()
+    gpu_tests_on_cpu.test_training_steps_on_the_gpu_operator_match_torch_autograd()
 
 
 def test_sign_range_test_walks_on_a_model_of_the_kernel(gpu_tests_on_cpu, monkeypatch):

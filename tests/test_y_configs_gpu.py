@@ -192,3 +192,23 @@ def test_model_blocks_on_the_gpu():
     assert cf.rel_err(out.detach(), out_ref.detach()) <= cc.FWD_TOL
     for a, b in zip(got, ref):
         assert cf.rel_err(a.grad, b.grad) <= cc.BWD_TOL
+
+
+def test_training_steps_on_the_gpu_operator_match_torch_autograd():
+    """tests/test_training_loop_cpu.py's loop (a two-layer transformer on the reference example's task, six Adam
+    steps) with l1attn_cuda.L1Attn in float64 on the GPU against the same graph on torch's autograd through the
+    closed form: weights and losses agree to rounding."""
+    print("case training loop", flush=True)
+    import l1attn_cuda
+    import test_training_loop_cpu as tl
+
+    class OnGpu(torch.nn.Module):  # the loop's tensors live on the CPU; only the operator's run on the GPU
+        def forward(self, q, k):
+            return l1attn_cuda.L1Attn()(q.to(DEV), k.to(DEV)).cpu()
+
+    net_a, loss_a = tl.train(OnGpu())
+    net_b, loss_b = tl.train(cf.dense_attn)
+    for la, lb in zip(loss_a, loss_b):
+        assert abs(la - lb) <= 1e-9 * max(1.0, abs(lb))
+    for pa, pb in zip(net_a.parameters(), net_b.parameters()):
+        assert cf.rel_err(pa.detach(), pb.detach()) <= 1e-9
