@@ -303,6 +303,17 @@ def check_hot_loops(asm_text, table=HOT_LOOPS):
 
 
 def build(verbose=False):
+    """Compile, check, link.  A build that fails a compile or a check leaves NO library behind: one from an
+    earlier build would no longer match the sources, and none that has not passed the checks may run."""
+    try:
+        return _build(verbose)
+    except BaseException:
+        if os.path.exists(LIB):
+            os.remove(LIB)
+        raise
+
+
+def _build(verbose):
     sys.path.insert(0, HERE)
     try:
         from isa_checks import check_forbidden  # travels with the sources on the build machine only

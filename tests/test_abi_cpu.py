@@ -259,7 +259,7 @@ _Z5kern2v: ; @k
         build.check_asm_sources({"fused.hip": 'void f()\n{\n\tasm("ds_read_b32 %0, %1" : "=v"(x) : "v"(o));\n}\n'})
 
 
-def test_build_runs_where_the_forbidden_instruction_list_does_not_travel(monkeypatch, capsys):
+def test_build_runs_where_the_forbidden_instruction_list_does_not_travel(monkeypatch, capsys, tmp_path):
     """isa_checks.py names instructions and stays on the build machine; build() must still import and run its
     other checks without it.  hipcc is replaced by a stand-in that fails at once, so only the start is walked."""
     import builtins
@@ -275,9 +275,14 @@ def test_build_runs_where_the_forbidden_instruction_list_does_not_travel(monkeyp
     monkeypatch.delitem(sys.modules, "isa_checks", raising=False)
     monkeypatch.setattr(builtins, "__import__", no_isa_checks)
     monkeypatch.setenv("HIPCC", "/bin/false")
+    # a failed build removes the library it would have replaced: point it at a stand-in file, not the real one
+    stale = tmp_path / "libl1attn_hip.so"
+    stale.write_bytes(b"left over from an earlier build")
+    monkeypatch.setattr(build, "LIB", str(stale))
     with pytest.raises(RuntimeError, match="hipcc failed"):
         build.build()
     assert "forbidden instructions is skipped" in capsys.readouterr().err
+    assert not stale.exists()
 
 
 def test_build_rejects_spills_in_the_hot_kernels():
