@@ -431,6 +431,23 @@ def cpu_baseline_sparse(mods, ncores):
         mods["l1attn_sparse_drv"].backward(d[3], d[0], d[1], d[2], coo, attn, dmx, True)
         dt = time.perf_counter() - t0
         out["reference_fp64"] = {"fwd_bwd_ms": dt * 1e3, "edges_per_s": E / dt, "cores": 1, "kind": "reference"}
+    # Configuration 5 (bidirectional, B1 T65536 H4 W64, about 1.08 M edges, longest dst segment 2049) on the CPU
+    # operator package only: the reference's extension would walk its O(dst_mxlen^2) softmax Jacobian loop
+    # (cpp/l1attn_sparse_bidi_drv.cpp:176-190) 65536 * 4 * 2049^2 = 1.1e12 times and hold 4.3 GB of float64 padding.
+    B, T, H, W = 1, 65536, 4, 64
+    co = workloads.powerlaw_graph(T, seed=1005)
+    coo, dmx, _ = _l1attn_cpu.expand_coo(co)
+    vf, vb, q, k = workloads.sparse_inputs(B, T, H, W, seed=1005, n=4)
+    dvo = torch.randn(B, T, H, W, generator=torch.Generator().manual_seed(1))
+    _l1attn_cpu.set_threads(ncores)
+    t0 = time.perf_counter()
+    vo, attn = _l1attn_cpu.bidi_forward(vf, vb, q, k, coo, dmx, True)
+    _l1attn_cpu.bidi_backward(dvo, vf, vb, q, k, coo, attn, dmx, True)
+    dt = time.perf_counter() - t0
+    _l1attn_cpu.set_threads(0)
+    out["config5_bidi_cpu_operator_package_fp32"] = {
+        "edges": int(co.shape[0]), "fwd_bwd_ms": dt * 1e3, "edges_per_s": int(co.shape[0]) / dt, "cores": ncores,
+        "note": "the reference's CPU extension is not timed here: O(dst_mxlen^2) Jacobian loop, 1.1e12 iterations"}
     return out
 
 
@@ -495,7 +512,7 @@ def cpu_baseline():
     except Exception as e:  # noqa: BLE001
         log("sparse CPU baseline not timed:", repr(e))
     return {
-        "sparse_config4": sparse,
+        "sparse": sparse,
         "cpu_operator_package_fp32": pkg,
         "value": 6 * N / dt / 1e9, "unit": "GOP/s", "cores": 1, "kind": kind,
         "sample": "dense fwd+bwd fp64, B=1 T=1024 H=16 W=64 (1/128 of the headline pair-elements), %.1f s" % dt,
