@@ -113,6 +113,26 @@ int l1attn_cpu_sparse_bidi_bwd_f64(const double* dvo, const double* vf, const do
                                    double* dvf, double* dvb, double* dq, double* dk, int64_t B, int64_t T, int64_t H,
                                    int64_t W, int64_t Wv, int64_t E, int64_t dst_mxlen, int use_softmax);
 
+/*
+ * Fused operator: dense L1 logits, softmax over the src tokens with the no-op zero logit, value sum, without the
+ * [B,S,T,H] logits -- the composition of example-setfind/setfind.py:128-136 (the reference has no single function
+ * for it; README.md:21 asks for it).  vo[b,t,h,:] = sum_s e^{a[s]} v[b,s,h,:] / (1 + sum_s e^{a[s]}),
+ * lse[b,t,h] = log(1 + sum_s e^{a[s]}) (lse may be NULL in the forward).  The backward takes the forward's vo and
+ * lse and returns dq, dk, dv; it holds no [T,T] tensor either (the logits are recomputed in two sweeps).
+ * q,k [B,T,H,W]; v, vo, dvo, dv [B,T,H,Wv].  The host twin of l1attn_fused_fwd_* / l1attn_fused_bwd_stage_* of the
+ * GPU library.
+ */
+int l1attn_cpu_fused_fwd_f32(const float* q, const float* k, const float* v, float* vo, float* lse,
+                             int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv);
+int l1attn_cpu_fused_fwd_f64(const double* q, const double* k, const double* v, double* vo, double* lse,
+                             int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv);
+int l1attn_cpu_fused_bwd_f32(const float* dvo, const float* q, const float* k, const float* v, const float* vo,
+                             const float* lse, float* dq, float* dk, float* dv,
+                             int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv);
+int l1attn_cpu_fused_bwd_f64(const double* dvo, const double* q, const double* k, const double* v, const double* vo,
+                             const double* lse, double* dq, double* dk, double* dv,
+                             int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv);
+
 #ifdef __cplusplus
 }
 #endif

@@ -45,6 +45,12 @@ def lib():
                 f.argtypes = [_c_p] * npre + [_c_i64] + [_c_p] * npost + [_c_i64] * 7 + [_c_i]
                 if name.endswith("_fwd"):
                     f.argtypes = f.argtypes + [_c_i]  # attn_zeroed
+            f = getattr(L, "l1attn_cpu_fused_fwd_" + sfx)
+            f.restype = _c_i
+            f.argtypes = [_c_p] * 5 + [_c_i64] * 5
+            f = getattr(L, "l1attn_cpu_fused_bwd_" + sfx)
+            f.restype = _c_i
+            f.argtypes = [_c_p] * 9 + [_c_i64] * 5
         _lib = L
     return _lib
 
@@ -217,3 +223,36 @@ def bidi_backward(dvo, vf, vb, q, k, coo, attn, dst_mxlen, use_softmax):
         _p(dvo), _p(vf), _p(vb), _p(q), _p(k), _p(coo), coo.shape[1], _p(attn), _p(dvf), _p(dvb), _p(dq), _p(dk),
         B, T, H, W, Wv, E, M, int(bool(use_softmax))), "l1attn_cpu_sparse_bidi_bwd_" + sfx)
     return [dvf, dvb, dq, dk]
+
+
+def fused_forward(q, k, v):
+    """Fused operator, forward -> [vo, lse]: softmax over src of the L1 logits with the no-op zero logit, times v,
+    without the [B,T,T,H] logits (example-setfind/setfind.py:128-136 in one call)."""
+    for x, n in ((q, "q"), (k, "k"), (v, "v")):
+        _check_input(x, n)
+    B, T, H, W = _dense_shapes(q, k)
+    if v.dim() != 4 or v.shape[:3] != q.shape[:3] or v.dtype != q.dtype:
+        raise RuntimeError("v must be [batch, n_ctx, n_heads, value width] with the dtype of q")
+    sfx = _sfx(q)
+    vo = torch.empty_like(v)
+    lse = torch.empty((B, T, H), dtype=q.dtype)
+    _check(getattr(lib(), "l1attn_cpu_fused_fwd_" + sfx)(_p(q), _p(k), _p(v), _p(vo), _p(lse), B, T, H, W, v.shape[3]),
+           "l1attn_cpu_fused_fwd_" + sfx)
+    return [vo, lse]
+
+
+def fused_backward(dvo, q, k, v, vo, lse):
+    """Backward of fused_forward -> [dq, dk, dv]."""
+    for x, n in ((dvo, "dvo"), (q, "q"), (k, "k"), (v, "v"), (vo, "vo"), (lse, "lse")):
+        _check_input(x, n)
+    B, T, H, W = _dense_shapes(q, k)
+    _same_as(dvo, v, "dvo", "v")
+    _same_as(vo, v, "vo", "v")
+    if v.dtype != q.dtype or tuple(lse.shape) != (B, T, H) or lse.dtype != q.dtype:
+        raise RuntimeError("v must have the dtype of q, and lse must be the [batch, n_ctx, n_heads] tensor the forward returned")
+    sfx = _sfx(q)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _check(getattr(lib(), "l1attn_cpu_fused_bwd_" + sfx)(
+        _p(dvo), _p(q), _p(k), _p(v), _p(vo), _p(lse), _p(dq), _p(dk), _p(dv), B, T, H, W, v.shape[3]),
+        "l1attn_cpu_fused_bwd_" + sfx)
+    return [dq, dk, dv]

@@ -183,4 +183,26 @@ int l1attn_cpu_expand_coo(const void* co, int co_bits, int64_t co_stride, int64_
 L1CPU_SPARSE(f32, float)
 L1CPU_SPARSE(f64, double)
 
+#define L1CPU_FUSED(SFX, F)                                                                                                  \
+	int l1attn_cpu_fused_fwd_##SFX(const F* q, const F* k, const F* v, F* vo, F* lse, int64_t B, int64_t T, int64_t H,       \
+	                               int64_t W, int64_t Wv)                                                                    \
+	{                                                                                                                        \
+		if (bad_dims(B, T, H, W) || Wv < 1) return L1ATTN_CPU_ERR_ARG;                                                       \
+		if (B * T * H == 0) return 0;                                                                                        \
+		if (!q || !k || !v || !vo) return L1ATTN_CPU_ERR_ARG;                                                                \
+		table().fused_fwd_##SFX(q, k, v, vo, lse, B, T, H, W, Wv, threads());                                                \
+		return 0;                                                                                                            \
+	}                                                                                                                        \
+	int l1attn_cpu_fused_bwd_##SFX(const F* dvo, const F* q, const F* k, const F* v, const F* vo, const F* lse, F* dq,       \
+	                               F* dk, F* dv, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv)                     \
+	{                                                                                                                        \
+		if (bad_dims(B, T, H, W) || Wv < 1) return L1ATTN_CPU_ERR_ARG;                                                       \
+		if (B * T * H == 0) return 0;                                                                                        \
+		if (!dvo || !q || !k || !v || !vo || !lse || !dq || !dk || !dv) return L1ATTN_CPU_ERR_ARG;                           \
+		table().fused_bwd_##SFX(dvo, q, k, v, vo, lse, dq, dk, dv, B, T, H, W, Wv, threads());                               \
+		return 0;                                                                                                            \
+	}
+L1CPU_FUSED(f32, float)
+L1CPU_FUSED(f64, double)
+
 }  // extern "C"

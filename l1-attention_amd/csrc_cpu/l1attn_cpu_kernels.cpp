@@ -106,6 +106,76 @@ void dense_bwd(const F* dA, const F* q, const F* k, F* dq, F* dk, int64_t B, int
 			}
 }
 
+// ------------------------------------------------------------------------------------------ fused
+// Dense logits, softmax over src with the no-op zero logit, value sum, without the [B,T,T,H] tensor:
+//   vo[b,t,h,:] = sum_s e^{a[s,t]} v[b,s,h,:] / (1 + sum_s e^{a[s,t]}),  lse = log(1 + sum_s e^{a[s,t]}).
+// Every logit is <= 0 and the no-op logit is 0, so no running maximum is needed.
+
+template <typename F>
+void fused_fwd(const F* q, const F* k, const F* v, F* vo, F* lse, int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv,
+               int nt)
+{
+	const F scale = (F)(-1.0 / std::sqrt((double)W));
+	const int64_t row = H * W, vrow = H * Wv;
+#pragma omp parallel for collapse(2) schedule(static) num_threads(nt)
+	for (int64_t b = 0; b < B; b++)
+		for (int64_t t = 0; t < T; t++) {
+			F* out = vo + (b * T + t) * vrow;
+			std::memset(out, 0, sizeof(F) * vrow);
+			for (int64_t h = 0; h < H; h++) {
+				const F* qt = q + (b * T + t) * row + h * W;
+				F den = 0;
+				for (int64_t s = 0; s < T; s++) {
+					const F p = std::exp(l1_row(qt, k + (b * T + s) * row + h * W, W) * scale);
+					den += p;
+					axpy(out + h * Wv, v + (b * T + s) * vrow + h * Wv, p, Wv);
+				}
+				const F inv = (F)1 / ((F)1 + den);
+				for (int64_t w = 0; w < Wv; w++) out[h * Wv + w] *= inv;
+				if (lse) lse[(b * T + t) * H + h] = std::log1p(den);
+			}
+		}
+}
+
+// Backward without any [T,T] tensor: with p = e^{a - lse[t]}, dp = v[s].dvo[t], S[t] = vo[t].dvo[t], the gradient of
+// a logit is da = p (dp - S[t]).  One sweep with the dst rows as owners (dq), one with the src rows as owners
+// (dk, dv); each recomputes the logits it needs.
+template <typename F>
+void fused_bwd(const F* dvo, const F* q, const F* k, const F* v, const F* vo, const F* lse, F* dq, F* dk, F* dv, int64_t B,
+               int64_t T, int64_t H, int64_t W, int64_t Wv, int nt)
+{
+	const F scale = (F)(-1.0 / std::sqrt((double)W));
+	const int64_t row = H * W, vrow = H * Wv;
+	std::vector<F> Sv((size_t)B * T * H);
+#pragma omp parallel for schedule(static) num_threads(nt)
+	for (int64_t i = 0; i < B * T * H; i++) Sv[i] = dot_row(vo + i * Wv, dvo + i * Wv, Wv);
+#pragma omp parallel for collapse(3) schedule(static) num_threads(nt)
+	for (int sweep = 0; sweep < 2; sweep++)
+		for (int64_t b = 0; b < B; b++)
+			for (int64_t r = 0; r < T; r++) {
+				F* gq = sweep == 0 ? dq + (b * T + r) * row : nullptr;
+				F* gk = sweep == 1 ? dk + (b * T + r) * row : nullptr;
+				F* gv = sweep == 1 ? dv + (b * T + r) * vrow : nullptr;
+				if (sweep == 0) std::memset(gq, 0, sizeof(F) * row);
+				else { std::memset(gk, 0, sizeof(F) * row); std::memset(gv, 0, sizeof(F) * vrow); }
+				for (int64_t o = 0; o < T; o++) {
+					const int64_t t = sweep == 0 ? r : o, s = sweep == 0 ? o : r;
+					for (int64_t h = 0; h < H; h++) {
+						const F* qt = q + (b * T + t) * row + h * W;
+						const F* ks = k + (b * T + s) * row + h * W;
+						const F* gt = dvo + (b * T + t) * vrow + h * Wv;
+						const F p = std::exp(l1_row(qt, ks, W) * scale - lse[(b * T + t) * H + h]);
+						const F da = p * (dot_row(v + (b * T + s) * vrow + h * Wv, gt, Wv) - Sv[(b * T + t) * H + h]);
+						if (sweep == 0) sign_axpy(gq + h * W, qt, ks, scale * da, W);
+						else {
+							sign_axpy(gk + h * W, qt, ks, -scale * da, W);
+							axpy(gv + h * Wv, gt, p, Wv);
+						}
+					}
+				}
+			}
+}
+
 // ----------------------------------------------------------------------------------- edge lists
 
 // Stable counting sort of the edges by column `col` of coo: ptr[T+1], order[E] (edge ids, original order
@@ -254,4 +324,6 @@ const L1CpuTable L1CPU_CAT(l1cpu_table_, L1CPU_NS) = {
     L1CPU_NS::sparse_fwd<float, true>,  L1CPU_NS::sparse_fwd<double, true>,
     L1CPU_NS::sparse_bwd<float, false>, L1CPU_NS::sparse_bwd<double, false>,
     L1CPU_NS::sparse_bwd<float, true>,  L1CPU_NS::sparse_bwd<double, true>,
+    L1CPU_NS::fused_fwd<float>,         L1CPU_NS::fused_fwd<double>,
+    L1CPU_NS::fused_bwd<float>,         L1CPU_NS::fused_bwd<double>,
 };

@@ -30,6 +30,14 @@ struct L1CpuTable {
 	void (*bidi_bwd_f64)(const double*, const double*, const double*, const double*, const double*, const int32_t*, int64_t,
 	                     const double*, double*, double*, double*, double*, int64_t, int64_t, int64_t, int64_t, int64_t,
 	                     int64_t, int64_t, bool, int);
+	void (*fused_fwd_f32)(const float*, const float*, const float*, float*, float*, int64_t, int64_t, int64_t, int64_t,
+	                      int64_t, int);
+	void (*fused_fwd_f64)(const double*, const double*, const double*, double*, double*, int64_t, int64_t, int64_t, int64_t,
+	                      int64_t, int);
+	void (*fused_bwd_f32)(const float*, const float*, const float*, const float*, const float*, const float*, float*, float*,
+	                      float*, int64_t, int64_t, int64_t, int64_t, int64_t, int);
+	void (*fused_bwd_f64)(const double*, const double*, const double*, const double*, const double*, const double*, double*,
+	                      double*, double*, int64_t, int64_t, int64_t, int64_t, int64_t, int);
 };
 
 extern const L1CpuTable l1cpu_table_l1cpu_generic;

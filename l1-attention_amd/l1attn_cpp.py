@@ -31,3 +31,30 @@ class L1Attn(nn.Module):
 
     def forward(self, q, k):
         return L1AttnFn.apply(q, k)
+
+
+class L1AttnFusedFn(Function):
+    """The host twin of l1attn_cuda.L1AttnFusedFn: softmax over the src tokens of the L1 logits with the no-op zero
+    logit, times v, without the [B,T,T,H] logits.  Equals
+    einsum('bsdh,bshw->bdhw', softmax(cat(L1Attn()(q,k), zeros), 1)[:, :-1], v), the composition of
+    example-setfind/setfind.py:128-136; the reference has no such function (README.md:21 asks for it)."""
+    @staticmethod
+    def forward(ctx, q, k, v):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        vo, lse = _drv.fused_forward(q, k, v)
+        ctx.save_for_backward(q, k, v, vo, lse)
+        return vo
+
+    @staticmethod
+    def backward(ctx, d_vo):
+        q, k, v, vo, lse = ctx.saved_tensors[:5]
+        d_q, d_k, d_v = _drv.fused_backward(d_vo.contiguous(), q, k, v, vo, lse)
+        return d_q, d_k, d_v
+
+
+class L1AttnFused(nn.Module):
+    def __init__(self):
+        super(L1AttnFused, self).__init__()
+
+    def forward(self, q, k, v):
+        return L1AttnFusedFn.apply(q, k, v)

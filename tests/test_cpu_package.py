@@ -52,7 +52,7 @@ def test_cpu_library_exports_every_declared_symbol_and_header_is_c():
     import _l1attn_cpu
     src = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
     names = sorted(set(re.findall(r"\b(l1attn_cpu_[a-z0-9_]+)\s*\(", src)))
-    assert len(names) == 15
+    assert len(names) == 19
     L = ctypes.CDLL(_l1attn_cpu._LIB_PATH)
     for n in names:
         assert hasattr(L, n), n
@@ -408,3 +408,59 @@ def test_live_reference_extension_when_built():
         for x, y in zip(l1attn_sparse_bidi_drv.backward(dvo, v, vb, q, k, coo, mine[1], dmx, sm),
                         mods["l1attn_sparse_bidi_drv"].backward(dvo, v, vb, q, k, coo, ref[1], dmx, sm)):
             assert cf.rel_err(x, y) <= F64_TOL
+
+
+# ------------------------------------------------------------------------------------------- fused
+
+@pytest.mark.parametrize("shape", [(2, 64, 4, 32, 32), (1, 100, 3, 64, 64), (2, 9, 3, 5, 5), (1, 37, 3, 32, 20),
+                                   (1, 1, 1, 1, 1), (2, 0, 3, 4, 4)])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_fused_operator_matches_the_oracle(shape, dtype):
+    """l1attn_cpp.L1AttnFused against the oracle's composition (the reference's dense CPU loop, then the no-op row,
+    softmax and einsum of example-setfind/setfind.py:128-136, differentiated by hand), against torch autograd through
+    the closed form where the value width differs, and against the same composition built on l1attn_cpp.L1Attn."""
+    l1, _, _ = _mods()
+    B, T, H, W, Wv = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    q, k = (torch.randn(B, T, H, W, generator=g, dtype=dtype) for _ in range(2))
+    v, dvo = (torch.randn(B, T, H, Wv, generator=g, dtype=dtype) for _ in range(2))
+    x = [t.clone().requires_grad_() for t in (q, k, v)]
+    vo = l1.L1AttnFused()(*x)
+    assert vo.shape == v.shape and vo.dtype == dtype
+    got = torch.autograd.grad(vo, x, dvo)
+    if T == 0:
+        return
+    ftol, gtol = (F64_TOL, 1e-11) if dtype == torch.float64 else (F32_FWD, F32_GRAD)
+    if W == Wv:
+        ref, ref_lse = oracle.fused_fwd(q.double(), k.double(), v.double())
+        rg = oracle.fused_bwd(dvo.double(), q.double(), k.double(), v.double())
+        import _l1attn_cpu as drv
+        assert cf.rel_err(drv.fused_forward(q, k, v)[1], ref_lse) <= ftol
+    else:
+        r = [t.double().requires_grad_() for t in (q, k, v)]
+        ref = cf.dense_then_value(*r, noop=True)
+        rg = torch.autograd.grad(ref, r, dvo.double())
+        ref = ref.detach()
+    assert cf.rel_err(vo.detach(), ref) <= ftol
+    for a, b in zip(got, rg):
+        assert cf.rel_err(a, b) <= gtol
+    # the same numbers from the unfused composition on the dense operator of this package
+    y = [t.clone().requires_grad_() for t in (q, k, v)]
+    a = l1.L1Attn()(y[0], y[1])
+    a = torch.cat((a, torch.zeros(B, 1, T, H, dtype=dtype)), 1)
+    comp = torch.einsum("bsdh,bshw->bdhw", torch.softmax(a, 1)[:, :T], y[2])
+    cg = torch.autograd.grad(comp, y, dvo)
+    assert cf.rel_err(vo.detach(), comp.detach().double()) <= 2 * ftol
+    for a_, b_ in zip(got, cg):
+        assert cf.rel_err(a_, b_.double()) <= 2 * gtol
+
+
+def test_fused_operator_gradcheck_and_sparse_equivalence():
+    l1, sp, _ = _mods()
+    g = torch.Generator().manual_seed(44)
+    q, k, v = (torch.randn(1, 5, 2, 6, dtype=torch.float64, generator=g).requires_grad_() for _ in range(3))
+    assert gradcheck(l1.L1AttnFusedFn.apply, (q, k, v), eps=1e-6, atol=1e-6, nondet_tol=0.0)
+    # equals sparse attention over the full cartesian edge list (python/l1attn_sparse.py:488-506)
+    T = 5
+    coo, dmx, _ = sp.expandCoo(torch.cartesian_prod(torch.arange(T), torch.arange(T)), warn=False)
+    assert cf.rel_err(l1.L1AttnFused()(q, k, v).detach(), sp.L1AttnSparse()(v, q, k, coo, dmx).detach()) <= F64_TOL
