@@ -235,6 +235,15 @@ def test_fixed_point_prepass_kernels_on_cpu(tmp_path):
     assert np.all(uq[1, :, 2] == 2 ** 31) and np.all(uk[1, :, 2] == 2 ** 31)
 
 
+@pytest.fixture(scope="module")
+def ranks_runner(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("emu_ranks") / "run_ranks")
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
+                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_ranks.cpp"), "-o", exe],
+                   check=True)
+    return exe
+
+
 def _reference_ranks(q, k):
     """rq, rk of one [B,T,H,W] pair by their definition, with numpy: per column, rk = 2 * #{k' < k} - 1/2 and
     rq = 2 * #{k' < q}, minus one where q ties with no k.  -0 and +0 are equal."""
@@ -255,15 +264,12 @@ def _reference_ranks(q, k):
 
 @pytest.mark.parametrize("shape", [(1, 4096, 1, 2), (1, 1000, 2, 2), (2, 300, 1, 3), (1, 2049, 1, 2), (1, 5000, 1, 1),
                                    (1, 1, 1, 5), (1, 513, 3, 1)])
-def test_merge_sort_column_ranks_on_cpu(tmp_path, shape):
+def test_merge_sort_column_ranks_on_cpu(tmp_path, shape, ranks_runner):
     """The merge-sort rank kernel (csrc/rank_sort.hip; registers, LDS and barriers only) under AddressSanitizer:
     every items-per-thread instantiation (T up to 512, 1024, 2048, 4096, 8192), ragged lengths (padding keys),
     planted ties between q and k, repeated k values, both zeros; ranks equal their definition exactly, and
     clamp(rq - rk, 0, 1) is 1, 1/2, 0 for q >, ==, < k on every pair of a column."""
-    exe = str(tmp_path / "run_ranks")
-    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
-                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_ranks.cpp"), "-o", exe],
-                   check=True)
+    exe = ranks_runner
     B, T, H, W = shape
     g = torch.Generator().manual_seed(sum(shape))
     q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))
