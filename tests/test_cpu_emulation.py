@@ -24,12 +24,8 @@ EMU = os.path.join(HERE, "cpu_emu")
 
 
 @pytest.fixture(scope="module")
-def runner(tmp_path_factory):
-    exe = str(tmp_path_factory.mktemp("emu") / "run_fused")
-    cmd = ["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
-           "-I", EMU, "-x", "c++", os.path.join(EMU, "run_fused.cpp"), "-o", exe]
-    subprocess.run(cmd, check=True)
-    return exe
+def runner(emu_fused):
+    return emu_fused
 
 
 @pytest.fixture(scope="module")
@@ -236,12 +232,8 @@ def test_fixed_point_prepass_kernels_on_cpu(tmp_path):
 
 
 @pytest.fixture(scope="module")
-def ranks_runner(tmp_path_factory):
-    exe = str(tmp_path_factory.mktemp("emu_ranks") / "run_ranks")
-    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
-                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_ranks.cpp"), "-o", exe],
-                   check=True)
-    return exe
+def ranks_runner(emu_ranks):
+    return emu_ranks
 
 
 def _reference_ranks(q, k):

@@ -31,12 +31,8 @@ pytestmark = pytest.mark.skipif(not os.path.exists(CLANG), reason="needs ROCm's 
 
 
 @pytest.fixture(scope="module")
-def runner(tmp_path_factory):
-    exe = str(tmp_path_factory.mktemp("emu_sparse") / "run_sparse")
-    subprocess.run([CLANG, "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
-                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_sparse.cpp"),
-                    "-o", exe], check=True)
-    return exe
+def runner(emu_sparse):
+    return emu_sparse
 
 
 def _plan_arrays(co, T):
