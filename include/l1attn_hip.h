@@ -170,7 +170,10 @@ int l1attn_fused_fwd_pipe_f32(const float* q, const float* k, const float* v, fl
  * and dv[b,s,h,:] = sum_t p[s,t] * dvo[b,t,h,:].  dq and dk are then l1attn_dense_bwd_* of (dA, q, k).
  * vo and lse are the forward's outputs.  dA is the only [B,T,T,H] tensor of the whole forward + backward
  * (the unfused composition of example-setfind/setfind.py:128-136 keeps the logits, the weights and the
- * gradients of both).  No counterpart in the reference.  Deterministic.  Shapes as l1attn_fused_fwd_*.
+ * gradients of both).  Batch entries are independent: a caller that cannot hold [B,T,T,H] calls this and
+ * l1attn_dense_bwd_* on slabs of batch entries (pointers advanced by whole entries, B = the slab's count) with one
+ * dA buffer of the slab's size reused in stream order, as the Python driver does (1 GiB by default).
+ * No counterpart in the reference.  Deterministic.  Shapes as l1attn_fused_fwd_*.
  */
 int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k, const float* v,
                                const float* vo, const float* lse, float* dA, float* dv,

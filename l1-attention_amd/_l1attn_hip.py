@@ -270,9 +270,32 @@ def dense_fused_forward(q, k, v, want_lse=False, pipelined=False):
     return [vo, lse]
 
 
+_fused_da_bytes = 1 << 30
+
+
+def set_fused_workspace_bytes(n):
+    """Most bytes the fused backward may hold as logit gradients at a time (default 1 GiB); returns the previous
+    setting.  The batch is worked through in slabs of as many entries as fit, never fewer than one."""
+    global _fused_da_bytes
+    if int(n) < 0:
+        raise ValueError("a byte count, got %r" % (n,))
+    old, _fused_da_bytes = _fused_da_bytes, int(n)
+    return old
+
+
+def fused_backward_slab(B, T, H, itemsize):
+    """Batch entries per slab of the fused backward: as many [T,T,H] blocks of logit gradients as fit the
+    workspace bound, at least one, at most B."""
+    per_entry = T * T * H * itemsize
+    return max(1, min(B, _fused_da_bytes // per_entry if per_entry else B))
+
+
 def dense_fused_backward(dvo, q, k, v, vo, lse):
-    """Backward of dense_fused_forward -> [dq, dk, dv].  Stage one writes dA [B,T,T,H] (the gradient of the
-    logits, from dvo and the forward's vo and lse) and dv; dq and dk are the dense backward of dA."""
+    """Backward of dense_fused_forward -> [dq, dk, dv].  Stage one writes dA (the gradient of the logits, from
+    dvo and the forward's vo and lse) and dv; dq and dk are the dense backward of dA.  Batch entries are
+    independent, so the batch goes through in slabs that share one dA buffer of [slab,T,T,H] (stream order
+    keeps a slab's readers ahead of the next slab's writer): the whole [B,T,T,H] tensor never exists, 1 GiB in place
+    of 8 GiB at B=8, T=4096, H=16 in float32.  A single batch entry beyond the bound still takes its [T,T,H]."""
     _require_experimental("fused", "the fused L1 attention operator")
     for x, n in ((dvo, "dvo"), (q, "q"), (k, "k"), (v, "v"), (vo, "vo"), (lse, "lse")):
         check_input(x, n)
@@ -287,14 +310,26 @@ def dense_fused_backward(dvo, q, k, v, vo, lse):
         raise RuntimeError("v must have the dtype and device of q, and lse must be the [batch, n_ctx, n_heads] "
                            "tensor the forward returned")
     sfx = sfx_of(q)
-    dA = torch.empty((B, T, T, H), dtype=q.dtype, device=q.device)
+    slab = fused_backward_slab(B, T, H, q.element_size())
+    dA = torch.empty((slab, T, T, H), dtype=q.dtype, device=q.device)
     dv = torch.empty_like(v)
-    with torch.cuda.device(q.device):
-        rc = getattr(lib(), "l1attn_fused_bwd_stage_" + sfx)(
-            ptr(dvo), ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse), ptr(dA), ptr(dv), B, T, H, W, v.shape[3],
-            stream_of(q))
-    check(rc, "l1attn_fused_bwd_stage_" + sfx)
-    dq, dk = dense_backward(dA, q, k)
+    if slab >= B:
+        with torch.cuda.device(q.device):
+            rc = getattr(lib(), "l1attn_fused_bwd_stage_" + sfx)(
+                ptr(dvo), ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse), ptr(dA), ptr(dv), B, T, H, W, v.shape[3],
+                stream_of(q))
+        check(rc, "l1attn_fused_bwd_stage_" + sfx)
+        dq, dk = dense_backward(dA, q, k)
+        return [dq, dk, dv]
+    dq, dk = torch.empty_like(q), torch.empty_like(k)
+    for b0 in range(0, B, slab):
+        b1 = min(B, b0 + slab)  # (a slice of leading batch entries of a contiguous tensor is contiguous)
+        with torch.cuda.device(q.device):
+            rc = getattr(lib(), "l1attn_fused_bwd_stage_" + sfx)(
+                ptr(dvo[b0:b1]), ptr(q[b0:b1]), ptr(k[b0:b1]), ptr(v[b0:b1]), ptr(vo[b0:b1]), ptr(lse[b0:b1]), ptr(dA),
+                ptr(dv[b0:b1]), b1 - b0, T, H, W, v.shape[3], stream_of(q))
+        check(rc, "l1attn_fused_bwd_stage_" + sfx)
+        dq[b0:b1], dk[b0:b1] = dense_backward(dA[:b1 - b0], q[b0:b1], k[b0:b1])
     return [dq, dk, dv]
 
 

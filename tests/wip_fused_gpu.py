@@ -206,6 +206,30 @@ def test_fused_backward_second_baseline_shape_vs_composition():
         assert cf.rel_err(g_.cpu(), r_.cpu().double()) <= 2e-4
 
 
+def test_fused_backward_in_batch_slabs_equals_the_whole_batch():
+    """The backward with a workspace bound that fits two of five batch entries (slabs of 2, 2, 1 through one
+    shared buffer) against the same call with room for all five: a batch entry's gradients do not depend on which
+    entries run beside it, so dv bitwise and dq, dk to 1e-6 of the largest gradient (their sums may be grouped
+    by launch geometry)."""
+    print("case fused backward slabs", flush=True)
+    import _l1attn_hip as drv
+    fz = _fused()
+    B, T, H, W = 5, 96, 4, 32
+    g = torch.Generator().manual_seed(77)
+    q, k, v, dvo = (torch.randn(B, T, H, W, generator=g).cuda() for _ in range(4))
+    vo, lse = drv.dense_fused_forward(q, k, v, want_lse=True)
+    whole = drv.dense_fused_backward(dvo, q, k, v, vo, lse)
+    old = drv.set_fused_workspace_bytes(2 * T * T * H * 4)
+    try:
+        assert drv.fused_backward_slab(B, T, H, 4) == 2
+        slabs = drv.dense_fused_backward(dvo, q, k, v, vo, lse)
+    finally:
+        drv.set_fused_workspace_bytes(old)
+    assert torch.equal(slabs[2], whole[2])
+    for a, b in zip(slabs[:2], whole[:2]):
+        assert cf.rel_err(a.cpu(), b.cpu().double()) <= 1e-6
+
+
 def test_probe_other_instructions_runs():
     """The instruction-rate probe launches for every op code and rejects an unknown one."""
     print("case probe ops", flush=True)
