@@ -26,6 +26,17 @@ for _p in (ROOT, os.path.join(ROOT, "l1-attention_amd"), os.path.join(ROOT, "tes
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
+# Where and on what the legs run.  The sizes are the benchmark's definition; they are names here only so that a
+# walk-through of this file without a GPU (tests/test_bench_dry_run_cpu.py) can shrink them.
+DEVICE = "cuda:0"
+HEADLINE = (8, 4096, 16, 64)          # B, T, H, W of the headline dense configuration
+SECOND = (16, 1024, 8, 64)            # the second dense configuration (extra legs)
+CONFIG4 = ((4, 4096, 8, 32), 64)      # sparse: B, T, H, W; degrees uniform in 1..64
+CONFIG5 = (1, 65536, 4, 64)           # bidirectional sparse, power-law degrees and self loops
+CPU_SAMPLE = (1, 1024, 16, 64)        # the dense sample the host baseline is timed on
+COPY_FLOATS = 1 << 28                 # 1 GiB: the copy the HBM counters are calibrated on
+SWEEP = {"B": 512, "H": 8, "T": (16, 32, 64, 128, 256), "W": (16, 32, 33, 64, 65, 96, 97, 128)}
+
 P_VALU_TOPS = 78.6     # 256 CU x 4 SIMD x 32 fp32 lanes/clk x 2.4 GHz; the 157.3 TFLOP/s datasheet figure counts FMA as 2
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
@@ -52,11 +63,15 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def _shape_name(shape):
+    return "B%d_T%d_H%d_W%d" % tuple(shape)
+
+
 def dense_headline(steps, warmup):
     import torch
     import l1attn_cuda
-    B, T, H, W = 8, 4096, 16, 64
-    dev = torch.device("cuda:0")
+    B, T, H, W = HEADLINE
+    dev = torch.device(DEVICE)
     import workloads
     q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
     q, k = q.to(dev).requires_grad_(), k.to(dev).requires_grad_()
@@ -127,11 +142,11 @@ def sparse_configs(skip_cpu, only=None):
     import l1attn_sparse_cuda as sp
     import l1attn_sparse_bidi_cuda as bi
     from oracle import oracle
-    dev = torch.device("cuda:0")
+    dev = torch.device(DEVICE)
     res = {}
     for name, bidi, (B, T, H, W), co in (
-            ("config4_uni", False, (4, 4096, 8, 32), lambda: workloads.uniform_degree_graph(4096, 64, seed=1004)),
-            ("config5_bidi", True, (1, 65536, 4, 64), lambda: workloads.powerlaw_graph(65536, seed=1005))):
+            ("config4_uni", False, CONFIG4[0], lambda: workloads.uniform_degree_graph(CONFIG4[0][1], CONFIG4[1], seed=1004)),
+            ("config5_bidi", True, CONFIG5, lambda: workloads.powerlaw_graph(CONFIG5[1], seed=1005))):
         if only and not name.startswith(only):
             continue
         co = co() if callable(co) else co
@@ -203,9 +218,9 @@ def extra_legs():
     import l1attn_sparse_bidi_cuda as bi
     import _l1attn_hip as drv
     drv.enable_experimental("fused", "rows16", "fixed")  # these legs exist to time exactly those paths
-    dev = torch.device("cuda:0")
+    dev = torch.device(DEVICE)
     res = {"fused_forward": {}, "sparse_16bit": {}}
-    for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
+    for name, (B, T, H, W) in ((_shape_name(SECOND), SECOND), (_shape_name(HEADLINE), HEADLINE)):
         q, k, v = (x.to(dev) for x in workloads.dense_inputs(B, T, H, W, seed=1002, with_v=True))
         fused, plain = l1attn_cuda.L1AttnFused(), l1attn_cuda.L1Attn()
 
@@ -256,8 +271,8 @@ def extra_legs():
         del q, k, v
         torch.cuda.empty_cache()
     for name, bidi, (B, T, H, W), co in (
-            ("config4_uni", False, (4, 4096, 8, 32), workloads.uniform_degree_graph(4096, 64, seed=1004)),
-            ("config5_bidi", True, (1, 65536, 4, 64), workloads.powerlaw_graph(65536, seed=1005))):
+            ("config4_uni", False, CONFIG4[0], workloads.uniform_degree_graph(CONFIG4[0][1], CONFIG4[1], seed=1004)),
+            ("config5_bidi", True, CONFIG5, workloads.powerlaw_graph(CONFIG5[1], seed=1005))):
         coo, dmx, smx = sp.expandCoo(co.to(dev), warn=False)
         x32 = [t.to(dev) for t in workloads.sparse_inputs(B, T, H, W, seed=1004 + bidi, n=4)]
         m = bi.L1AttnSparseBidi() if bidi else sp.L1AttnSparse()
@@ -279,7 +294,7 @@ def extra_legs():
         res["sparse_16bit"][name] = row
         log(name, json.dumps(row))
     res["fixed_point_forward"] = {}
-    for name, (B, T, H, W) in (("B16_T1024_H8_W64", (16, 1024, 8, 64)), ("B8_T4096_H16_W64", (8, 4096, 16, 64))):
+    for name, (B, T, H, W) in ((_shape_name(SECOND), SECOND), (_shape_name(HEADLINE), HEADLINE)):
         q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
         q, k = q.to(dev), k.to(dev)
         ms32 = time_gpu(lambda: drv.dense_forward(q, k), 5)
@@ -296,17 +311,17 @@ def extra_legs():
         torch.cuda.empty_cache()
     res["instruction_rates"] = instruction_rates()
     # column ranks of the long-sequence backward: library block radix sort against the merge sort of rank_sort.hip
-    B, T, H, W = 8, 4096, 16, 64
+    B, T, H, W = HEADLINE
     q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
     q, k = q.to(dev), k.to(dev)
     rq, rk = torch.empty_like(q), torch.empty_like(k)
     L, st = drv.lib(), drv.stream_of(q)
-    res["column_ranks_B8_T4096_H16_W64"] = {
+    res["column_ranks_" + _shape_name(HEADLINE)] = {
         "library_radix_sort_ms": time_gpu(lambda: L.l1attn_dense_column_ranks_f32(
             drv.ptr(q), drv.ptr(k), drv.ptr(rq), drv.ptr(rk), B, T, H, W, st), 10),
         "merge_sort_ms": time_gpu(lambda: L.l1attn_dense_column_ranks_merge_f32(
             drv.ptr(q), drv.ptr(k), drv.ptr(rq), drv.ptr(rk), B, T, H, W, st), 10)}
-    log(json.dumps(res["column_ranks_B8_T4096_H16_W64"]))
+    log(json.dumps(res["column_ranks_" + _shape_name(HEADLINE)]))
     return res
 
 
@@ -317,7 +332,7 @@ def instruction_rates():
     import _l1attn_hip as drv
     L = drv.lib()
     blocks, iters = 256, 4000
-    out = torch.empty(blocks * 512, dtype=torch.float32, device="cuda:0")
+    out = torch.empty(blocks * 512, dtype=torch.float32, device=DEVICE)
     st = drv.stream_of(out)
     names = {0: "v_fmac_f32", 1: "v_sad_u32 (VGPR operands)", 2: "v_sad_u32 (SGPR operand)",
              3: "v_sub_f32 + v_add_f32 |x| (two instructions per step)"}
@@ -345,11 +360,11 @@ def reference_sweep(num_runs=10):
     and each cell also reports algorithmic Tops/s.  One JSON line per cell on stdout, and the list as return value."""
     import torch
     import l1attn_cuda
-    dev = torch.device("cuda:0")
-    B, H = 512, 8
+    dev = torch.device(DEVICE)
+    B, H = SWEEP["B"], SWEEP["H"]
     rows = []
-    for T in (16, 32, 64, 128, 256):
-        for W in (16, 32, 33, 64, 65, 96, 97, 128):
+    for T in SWEEP["T"]:
+        for W in SWEEP["W"]:
             g = torch.Generator(device=dev).manual_seed(1000 + T * 1000 + W)
             q = torch.randn(B, T, H, W, device=dev, generator=g).requires_grad_()
             k = torch.randn(B, T, H, W, device=dev, generator=g).requires_grad_()
@@ -386,7 +401,7 @@ def valu_probe():
     import _l1attn_hip as drv
     L = drv.lib()
     blocks, iters = 256, 4000
-    out = torch.empty(blocks * 512, dtype=torch.float32, device="cuda:0")
+    out = torch.empty(blocks * 512, dtype=torch.float32, device=DEVICE)
     st = drv.stream_of(out)
     assert L.l1attn_probe_valu(drv.ptr(out), blocks, 100, st) == 0
     torch.cuda.synchronize()
@@ -409,8 +424,8 @@ def cpu_baseline_sparse(mods, ncores):
     import torch
     import workloads
     import _l1attn_cpu
-    B, T, H, W = 4, 4096, 8, 32
-    co = workloads.uniform_degree_graph(T, 64, seed=1004)
+    (B, T, H, W), max_degree = CONFIG4
+    co = workloads.uniform_degree_graph(T, max_degree, seed=1004)
     coo, dmx, _ = _l1attn_cpu.expand_coo(co)
     v, _, q, k = workloads.sparse_inputs(B, T, H, W, seed=1004, n=4)
     dvo = torch.randn(B, T, H, W, generator=torch.Generator().manual_seed(1))
@@ -434,7 +449,7 @@ def cpu_baseline_sparse(mods, ncores):
     # Configuration 5 (bidirectional, B1 T65536 H4 W64, about 1.08 M edges, longest dst segment 2049) on the CPU
     # operator package only: the reference's extension would walk its O(dst_mxlen^2) softmax Jacobian loop
     # (cpp/l1attn_sparse_bidi_drv.cpp:176-190) 65536 * 4 * 2049^2 = 1.1e12 times and hold 4.3 GB of float64 padding.
-    B, T, H, W = 1, 65536, 4, 64
+    B, T, H, W = CONFIG5
     co = workloads.powerlaw_graph(T, seed=1005)
     coo, dmx, _ = _l1attn_cpu.expand_coo(co)
     vf, vb, q, k = workloads.sparse_inputs(B, T, H, W, seed=1005, n=4)
@@ -458,7 +473,7 @@ def cpu_baseline():
     import torch
     import workloads
     from oracle import oracle
-    B, T, H, W = 1, 1024, 16, 64
+    B, T, H, W = CPU_SAMPLE
     q, k, _ = workloads.dense_inputs(B, T, H, W, seed=1002)
     q, k = q.double(), k.double()
     dA = torch.randn(B, T, T, H, generator=torch.Generator().manual_seed(1002), dtype=torch.float64)
@@ -515,7 +530,8 @@ def cpu_baseline():
         "sparse": sparse,
         "cpu_operator_package_fp32": pkg,
         "value": 6 * N / dt / 1e9, "unit": "GOP/s", "cores": 1, "kind": kind,
-        "sample": "dense fwd+bwd fp64, B=1 T=1024 H=16 W=64 (1/128 of the headline pair-elements), %.1f s" % dt,
+        "sample": "dense fwd+bwd fp64, B=%d T=%d H=%d W=%d (1/%d of the headline pair-elements), %.1f s"
+                  % (B, T, H, W, round(HEADLINE[0] * HEADLINE[1] ** 2 * HEADLINE[2] * HEADLINE[3] / N), dt),
         "port_fp32_openmp": {"value": 6 * N / dt_mt / 1e9, "unit": "GOP/s", "cores": ncores,
                              "note": "OpenMP over (batch, head) of the C restatement"},
     }
@@ -560,7 +576,7 @@ def main():
     _l1attn_hip.lib()  # fail here, loudly, if the HIP library is not built
 
     if args.copy_calibration:
-        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        src = torch.empty(COPY_FLOATS, dtype=torch.float32, device=DEVICE).normal_()
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
@@ -600,9 +616,10 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": d["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "dense L1Attn fwd+bwd, q,k fp32 [B=8,T=4096,H=16,W=64], dA [8,4096,4096,16] "
-                               "(BASELINE.json configs[2], the headline dense configuration)",
-                   "B": 8, "T": 4096, "H": 16, "W": 64},
+        "config": {"workload": "dense L1Attn fwd+bwd, q,k fp32 [B=%d,T=%d,H=%d,W=%d], dA [%d,%d,%d,%d] "
+                               "(BASELINE.json configs[2], the headline dense configuration)"
+                               % (d["B"], d["T"], d["H"], d["W"], d["B"], d["T"], d["T"], d["H"]),
+                   "B": d["B"], "T": d["T"], "H": d["H"], "W": d["W"]},
         "frac_of_fp32_valu_peak": d["frac_of_valu_peak"],
         "valu_probe": _guarded(valu_probe),
         "dense": d,
