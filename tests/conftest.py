@@ -28,28 +28,51 @@ EMU = os.path.join(ROOT, "tests", "cpu_emu")
 CLANG = "/opt/rocm/llvm/bin/clang++"
 
 
-def _emu_runner(tmp_path_factory, name, cxx):
-    """The CPU build of one kernel file's runner (tests/cpu_emu/run_<name>.cpp) under AddressSanitizer and
-    UndefinedBehaviorSanitizer; built once per session, every emulation test module shares it."""
-    exe = str(tmp_path_factory.mktemp("emu_" + name) / ("run_" + name))
-    subprocess.run([cxx, "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
-                    "-fno-sanitize-recover=all", "-I", EMU, "-x", "c++", os.path.join(EMU, "run_%s.cpp" % name), "-o", exe],
-                   check=True)
+RUNNERS = {"fused": "g++", "sparse": CLANG, "ranks": "g++", "dense": "g++"}
+
+
+@pytest.fixture(scope="session")
+def _emu_builds(tmp_path_factory):
+    """The CPU builds of the kernel files' runners (tests/cpu_emu/run_<name>.cpp) under AddressSanitizer and
+    UndefinedBehaviorSanitizer, started side by side at the first request and shared by every emulation test
+    module of the session.  Line tables only: enough for a sanitizer report to name the line."""
+    d = tmp_path_factory.mktemp("emu")
+    jobs = {}
+    for name, cxx in RUNNERS.items():
+        if cxx == CLANG and not os.path.exists(CLANG):
+            continue
+        exe = str(d / ("run_" + name))
+        lines = "-gline-tables-only" if cxx == CLANG else "-g1"
+        cmd = [cxx, "-std=c++20", "-O1", lines, "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+               "-I", EMU, "-x", "c++", os.path.join(EMU, "run_%s.cpp" % name), "-o", exe]
+        jobs[name] = (exe, cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    return jobs
+
+
+def _emu_runner(builds, name):
+    if name not in builds:
+        pytest.skip("needs ROCm's clang++ as host compiler")
+    exe, cmd, proc = builds[name]
+    text, _ = proc.communicate() if proc.returncode is None else ("", None)
+    assert proc.returncode == 0, "%s\n%s" % (" ".join(cmd), text)
     return exe
 
 
 @pytest.fixture(scope="session")
-def emu_fused(tmp_path_factory):
-    return _emu_runner(tmp_path_factory, "fused", "g++")
+def emu_fused(_emu_builds):
+    return _emu_runner(_emu_builds, "fused")
 
 
 @pytest.fixture(scope="session")
-def emu_sparse(tmp_path_factory):
-    if not os.path.exists(CLANG):
-        pytest.skip("needs ROCm's clang++ as host compiler")
-    return _emu_runner(tmp_path_factory, "sparse", CLANG)
+def emu_sparse(_emu_builds):
+    return _emu_runner(_emu_builds, "sparse")
 
 
 @pytest.fixture(scope="session")
-def emu_ranks(tmp_path_factory):
-    return _emu_runner(tmp_path_factory, "ranks", "g++")
+def emu_ranks(_emu_builds):
+    return _emu_runner(_emu_builds, "ranks")
+
+
+@pytest.fixture(scope="session")
+def emu_dense(_emu_builds):
+    return _emu_runner(_emu_builds, "dense")

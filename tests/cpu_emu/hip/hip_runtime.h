@@ -1,5 +1,6 @@
 // TEST INFRASTRUCTURE: a host-only stand-in for the few HIP constructs that the library's simpler
-// kernels use (no cross-lane operations, no inline assembly), so that such a kernel can be compiled
+// kernels use (inline assembly only behind the library's two helper headers, for which the runners hold
+// stand-ins), so that such a kernel can be compiled
 // with g++ and run on the CPU under AddressSanitizer: every GPU thread of a workgroup is an OS thread,
 // __syncthreads() is a barrier among them, __shared__ arrays are static storage (workgroups run one
 // after the other).  It checks a kernel's index arithmetic, clamps, store predicates, LDS indexing,
@@ -57,6 +58,7 @@ inline std::unique_ptr<std::barrier<>> wg_barrier;  // the running workgroup's _
 // bracketed by a barrier among the wave's 64 threads.
 inline std::vector<std::unique_ptr<std::barrier<>>> wave_barrier;
 inline std::vector<double> wave_slots;  // 64 exchange slots per wave
+inline unsigned char* dynamic_lds = nullptr;  // the launch's dynamically sized LDS array, exactly `lds` bytes
 inline unsigned flat_tid() { return threadIdx_.x + blockDim_.x * (threadIdx_.y + blockDim_.y * threadIdx_.z); }
 inline void wave_sync() { wave_barrier[flat_tid() >> 6]->arrive_and_wait(); }
 }
@@ -69,8 +71,11 @@ using std::min;
 using std::max;
 
 #include <string.h>
+#include <stdlib.h>
 static inline unsigned __float_as_uint(float x) { unsigned u; memcpy(&u, &x, 4); return u; }
 static inline float __uint_as_float(unsigned u) { float x; memcpy(&x, &u, 4); return x; }
+static inline int __float_as_int(float x) { int u; memcpy(&u, &x, 4); return u; }
+static inline float __int_as_float(int u) { float x; memcpy(&x, &u, 4); return x; }
 
 // value of the wave's first active lane; the kernels built here only pass wave-uniform values
 static inline int __builtin_amdgcn_readfirstlane(int x) { return x; }
@@ -85,6 +90,44 @@ static inline T __shfl_xor(T x, int lane_mask)
 	emu::wave_sync();
 	return r;
 }
+// DPP row shift right by n (control 0x110 + n) with out-of-row lanes reading zero: lane l of each aligned group
+// of sixteen receives the value of lane l - n of the same group.  Every lane of the wave must call it.
+static inline int emu_dpp_row_shr(int src, int ctrl)
+{
+	const unsigned tid = emu::flat_tid(), n = (unsigned)ctrl & 15u;
+	emu::wave_slots[tid] = (double)src;
+	emu::wave_sync();
+	const int r = ((tid & 15u) >= n) ? (int)emu::wave_slots[tid - n] : 0;
+	emu::wave_sync();
+	return r;
+}
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound_ctrl) \
+	(static_cast<void>(sizeof(char[((ctrl) > 0x110 && (ctrl) < 0x120 && (bound_ctrl)) ? 1 : -1])), emu_dpp_row_shr(src, ctrl))
+// Raw buffer access: base + per-lane byte offset + uniform byte offset, both unsigned 32-bit; the library's
+// descriptors are unbounded below 4 GiB, so an offset sum that reaches 2^32 would be dropped on the GPU: abort here.
+struct __amdgpu_buffer_rsrc_t { char* base; };
+static inline char* emu_buf_at(__amdgpu_buffer_rsrc_t r, int v, int s)
+{
+	const uint64_t off = (uint64_t)(unsigned)v + (uint64_t)(unsigned)s;
+	if (off >= ((uint64_t)1 << 32)) abort();
+	return r.base + off;
+}
+static inline unsigned emu_buf_load(__amdgpu_buffer_rsrc_t r, int v, int s) { unsigned u; memcpy(&u, emu_buf_at(r, v, s), 4); return u; }
+static inline void emu_buf_store(unsigned u, __amdgpu_buffer_rsrc_t r, int v, int s) { memcpy(emu_buf_at(r, v, s), &u, 4); }
+static inline void emu_buf_fadd(float x, __amdgpu_buffer_rsrc_t r, int v, int s)
+{
+	float y; memcpy(&y, emu_buf_at(r, v, s), 4); y += x; memcpy(emu_buf_at(r, v, s), &y, 4);
+}
+#define __builtin_amdgcn_make_buffer_rsrc(p, stride, num, flags) (__amdgpu_buffer_rsrc_t{(char*)(p)})
+#define __builtin_amdgcn_raw_buffer_load_b32(r, v, s, aux) emu_buf_load(r, v, s)
+#define __builtin_amdgcn_raw_buffer_store_b32(u, r, v, s, aux) emu_buf_store(u, r, v, s)
+#define __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(x, r, v, s, aux) emu_buf_fadd(x, r, v, s)
+// scheduling and wait hints have no meaning here
+#define __builtin_amdgcn_s_waitcnt(x) ((void)0)
+#ifndef __clang__
+#define __builtin_nontemporal_store(v, p) (*(p) = (v))
+#define __builtin_nontemporal_load(p) (*(p))
+#endif
 // Memory fences order a wave's own stores before its own later loads from other lanes: lockstep lanes need
 // nothing more on the GPU, OS threads need a barrier among the wave.
 #define __builtin_amdgcn_fence(order, scope) emu::wave_sync()
@@ -92,8 +135,11 @@ static inline T __shfl_xor(T x, int lane_mask)
 static inline void __syncthreads() { emu::wg_barrier->arrive_and_wait(); }
 
 template <typename K, typename... A>
-static inline void emu_launch(K kernel, dim3 grid, dim3 block, A... args)
+static inline void emu_launch(K kernel, dim3 grid, dim3 block, size_t lds, A... args)
 {
+	// exactly sized, so that AddressSanitizer sees an access beyond the launch's LDS size
+	std::unique_ptr<unsigned char[]> lds_mem(lds ? new unsigned char[lds] : nullptr);
+	emu::dynamic_lds = lds_mem.get();
 	emu::gridDim_ = grid;
 	emu::blockDim_ = block;
 	const unsigned nt = block.x * block.y * block.z;
@@ -121,4 +167,4 @@ static inline void emu_launch(K kernel, dim3 grid, dim3 block, A... args)
 	emu::n_threads_run += (long)nt * nblocks;
 }
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
-	emu_launch(kernel, dim3(grid), dim3(block), __VA_ARGS__)
+	emu_launch(kernel, dim3(grid), dim3(block), (size_t)(lds), __VA_ARGS__)

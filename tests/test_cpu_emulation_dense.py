@@ -1,0 +1,172 @@
+"""CPU-only: the dense operator's kernel source (csrc/dense.hip: forward, backward, fixed-point forward) compiled
+for the host and run through the library's own entry points, against the oracle.
+
+tests/cpu_emu/run_dense.cpp includes the kernel file as it is.  GPU threads are OS threads, the LDS barrier is a
+barrier among them, DPP row shifts and raw buffer accesses are host functions, and the two headers that hold the
+library's hand-written instructions (csrc/sload.h, csrc/gfx950.h) are replaced by stand-ins that compute what those
+instructions compute (the scalar prefetch delivers at its wait and poisons at its load).  Everything else -- the
+host logic that picks kernels, grids, tile plans and workspace, every index, clamp, predicate and LDS offset of the
+kernels -- is the product's.  Buffers and the launch's LDS have their exact sizes under AddressSanitizer, outputs
+start as NaN (an element never written fails the comparison), and one build runs under ThreadSanitizer (a missing
+barrier is a data race).  This says nothing about timing, register allocation or the instruction encodings.
+
+The 512-thread tile kernels are chosen by the library from 1024 tokens and a few thousand workgroups on; the runner
+can build their plan for any length ("wide"), which is how they are walked here at 100 to 260 tokens."""
+import os
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+import closed_forms as cf
+from oracle import oracle
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+EMU = os.path.join(HERE, "cpu_emu")
+ENV = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0",
+           TSAN_OPTIONS="halt_on_error=1 report_signal_unsafe=0")
+
+
+def _run(exe, d, shape, mode="f32", extra=(), seed=0, ties=False, scale=1.0):
+    """-> dict with attn, dq, dk (as far as the mode has them), plan, and the inputs."""
+    B, T, H, W = shape
+    dt = torch.float64 if mode == "f64" else torch.float32
+    g = torch.Generator().manual_seed(seed)
+    q, k = (torch.randn(B, T, H, W, generator=g, dtype=dt) * scale for _ in range(2))
+    if ties:  # half-integers: exact ties between q and k, and among the k of a column
+        q, k = torch.round(q * 2) / 2, torch.round(k * 2) / 2
+    dA = torch.randn(B, T, T, H, generator=g, dtype=dt)
+    fin, fout = str(d / "in.bin"), str(d / "out.bin")
+    with open(fin, "wb") as f:
+        f.write(struct.pack("4q", B, T, H, W))
+        for x in (q, k, dA):
+            f.write(x.numpy().tobytes())
+    r = subprocess.run([exe, fin, fout, mode] + [str(x) for x in extra], env=ENV, capture_output=True, text=True)
+    assert r.returncode == 0, (shape, mode, extra, r.returncode, r.stderr[-3000:])
+    raw = open(fout, "rb").read()
+    npdt = np.float64 if mode == "f64" else np.float32
+    it, na, n = np.dtype(npdt).itemsize, B * T * T * H, B * T * H * W
+    out = {"q": q, "k": k, "dA": dA, "attn": torch.from_numpy(np.frombuffer(raw, npdt, na).reshape(B, T, T, H).copy())}
+    off = na * it
+    if mode != "fixed":
+        out["dq"] = torch.from_numpy(np.frombuffer(raw, npdt, n, off).reshape(B, T, H, W).copy())
+        out["dk"] = torch.from_numpy(np.frombuffer(raw, npdt, n, off + n * it).reshape(B, T, H, W).copy())
+        off += 2 * n * it
+    assert len(raw) == off + 16 * 8
+    keys = ("tiled", "wide", "rank", "branch_free", "threads", "n_cc", "n_tt", "tt_rows", "per", "group", "n_groups")
+    out["plan"] = dict(zip(keys, np.frombuffer(raw, np.int64, 16, off).tolist()))
+    return out
+
+
+def _check(r, fwd_tol, bwd_tol):
+    q, k, dA = (r[n].double() for n in ("q", "k", "dA"))
+    assert cf.rel_err(r["attn"], oracle.dense_fwd(q, k)) <= fwd_tol      # (NaN, i.e. an unwritten element, fails too)
+    if "dq" in r:
+        rdq, rdk = oracle.dense_bwd(dA, q, k)
+        assert cf.rel_err(r["dq"], rdq) <= bwd_tol and cf.rel_err(r["dk"], rdk) <= bwd_tol
+
+
+@pytest.fixture(scope="module")
+def runner(emu_dense):
+    return emu_dense
+
+
+# shape, and what it is there for
+LIBRARY_CASES = [
+    ((2, 64, 4, 32), "first baseline configuration: pipelined forward 32, 32-token tiles"),
+    ((1, 3, 2, 7), "the reference's test shape: one-workgroup forward, untiled backward"),
+    ((2, 17, 3, 5), "short odd sequence, H*W < 32"),
+    ((1, 70, 2, 9), "no multiple of anything: grid-stride forward, untiled backward"),
+    ((1, 40, 2, 7), "width 7 on zero-padded rows of 16"),
+    ((2, 100, 3, 33), "width 33 on padded rows of 48, ragged last tile, heads straddling column chunks"),
+    ((1, 50, 2, 65), "width 65 on padded rows of 80"),
+    ((1, 40, 1, 100), "width 100 on padded rows of 128 (half-head kernel)"),
+    ((1, 70, 20, 16), "twenty heads: two head groups in the forward, eight staged values per thread"),
+    ((1, 40, 16, 8), "sixteen staged values per thread"),
+    ((1, 64, 4, 48), "forward 48"),
+    ((1, 96, 2, 80), "forward 80"),
+    ((1, 64, 3, 96), "pipelined forward 96"),
+    ((1, 64, 2, 112), "forward 112"),
+    ((1, 64, 2, 128), "width 128 as two half-heads of the pipelined forward 64"),
+    ((2, 33, 1, 320), "width beyond the tiled forward"),
+    ((1, 72, 16, 64), "headline head geometry: sixteen waves per forward workgroup, two column chunks"),
+    ((1, 264, 2, 64), "several src chunks per dst tile in the forward"),
+]
+
+
+@pytest.mark.parametrize("shape,why", LIBRARY_CASES, ids=[str(c[0]) for c in LIBRARY_CASES])
+def test_dense_kernels_as_the_library_picks_them(runner, tmp_path, shape, why):
+    _check(_run(runner, tmp_path, shape, seed=sum(shape)), 1e-5, 1e-4)
+
+
+def test_the_cases_reach_the_kernel_families(runner, tmp_path):
+    """The plans of the shapes above, so that a change of the host logic that moves a case to another kernel
+    (and silently thins this file's coverage) is noticed."""
+    tiled = {s: _run(runner, tmp_path, s)["plan"] for s in [(2, 64, 4, 32), (1, 70, 20, 16), (1, 40, 16, 8), (1, 3, 2, 7)]}
+    assert [tiled[s]["tiled"] for s in tiled] == [1, 1, 1, 0]
+    assert [tiled[s]["per"] for s in list(tiled)[:3]] == [4, 8, 16] and tiled[(2, 64, 4, 32)]["tt_rows"] == 32
+
+
+def test_dense_float64_and_ties(runner, tmp_path):
+    for shape in ((2, 20, 3, 5), (1, 70, 2, 9)):
+        _check(_run(runner, tmp_path, shape, mode="f64", seed=4), 1e-13, 1e-13)
+    r = _run(runner, tmp_path, (2, 64, 4, 32), ties=True, seed=9)
+    assert float((r["q"][:, :, None] == r["k"][:, None]).float().mean()) > 0.1  # sign(0) = 0 matters here
+    _check(r, 1e-6, 1e-5)
+    _check(_run(runner, tmp_path, (1, 33, 2, 7), ties=True, seed=9), 1e-6, 1e-5)  # untiled kernels, exact compares
+
+
+WIDE_CASES = [
+    # shape, tile height, rank form, tiles per workgroup, half-integer inputs
+    ((2, 128, 2, 64), 64, 0, 1, False),     # branch-free step loop, one tile per workgroup
+    ((2, 128, 2, 64), 64, 1, 1, True),      # ... on column ranks
+    ((3, 128, 8, 64), 64, 0, 2, True),      # grouped tiles: the later tile adds to the stored partial; batch loop
+    ((3, 128, 2, 64), 64, 1, 2, False),
+    ((1, 256, 4, 64), 64, 1, 4, False),     # the headline instantiation <64,512,4,rank,grouped,branch-free>
+    ((1, 100, 3, 33), 64, 0, 1, False),     # general form: ragged tile, idle lanes shadowing a column
+    ((1, 136, 4, 64), 64, 1, 1, True),      # general form on ranks: T not a multiple of 64
+    ((1, 140, 16, 32), 64, 0, 1, False),    # eight staged values per thread
+    ((1, 100, 8, 64), 72, 1, 1, True),
+    ((1, 150, 8, 64), 80, 1, 1, False),
+    ((1, 150, 8, 64), 88, 0, 1, False),
+    ((1, 90, 16, 64), 72, 0, 1, False),     # two column chunks
+    ((1, 100, 5, 96), 64, 1, 1, False),     # heads of 96 columns: a chunk of 480 columns touches five heads
+]
+
+
+@pytest.mark.parametrize("shape,tt,rank,group,ties", WIDE_CASES, ids=["%s-tt%d-r%d-g%d" % (c[0], c[1], c[2], c[3]) for c in WIDE_CASES])
+def test_dense_backward_wide_tile_kernels(runner, tmp_path, shape, tt, rank, group, ties):
+    # (the rank form sums 2*hv*g and subtracts the row and column sums of g: a few more roundings than the oracle's sum)
+    _check(_run(runner, tmp_path, shape, extra=("wide", tt, rank, group), seed=sum(shape) + tt, ties=ties), 1e-5, 1e-4)
+
+
+def test_plans_outside_the_kernels_limits_are_refused(runner, tmp_path):
+    """The runner's plan builder mirrors the library's limits: sixteen lanes per staged (src row, head) in the rank
+    form, at most eight staged values per thread."""
+    for shape, extra in (((1, 100, 3, 33), ("wide", 72, 1, 1)), ((1, 150, 4, 32), ("wide", 88, 0, 1))):
+        with pytest.raises(AssertionError, match=r"wide.*, 4, "):
+            _run(runner, tmp_path, shape, extra=extra)
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 4, 32), (1, 100, 3, 64), (2, 40, 2, 64)])
+def test_fixed_point_forward_kernel(runner, tmp_path, shape):
+    """dense_fwd_f32_pipe<W, true> behind both pre-passes: the 24-bit grid per (batch, head) keeps the logits
+    within 1e-5 of the float64 oracle on N(0,1) inputs."""
+    _check(_run(runner, tmp_path, shape, mode="fixed", seed=sum(shape)), 1e-5, None)
+
+
+def test_dense_kernels_under_thread_sanitizer(tmp_path_factory):
+    """A barrier missing between a step's LDS writes and reads, or between two steps, is a data race here.
+    Shapes with whole column chunks only: lanes beyond the last column deliberately redo the chunk's first
+    column and store the same bits to the same address, which ThreadSanitizer rightly calls a race."""
+    d = tmp_path_factory.mktemp("emu_dense_tsan")
+    exe = str(d / "run_dense")
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=thread", "-I", EMU, "-x", "c++",
+                    os.path.join(EMU, "run_dense.cpp"), "-o", exe], check=True)
+    _check(_run(exe, d, (1, 64, 4, 32), seed=1), 1e-5, 1e-4)
+    _check(_run(exe, d, (1, 70, 3, 64), seed=2), 1e-5, 1e-4)
+    _check(_run(exe, d, (1, 128, 4, 64), extra=("wide", 64, 1, 2), seed=3), 1e-5, 1e-4)
+    _check(_run(exe, d, (1, 136, 2, 64), extra=("wide", 72, 0, 1), seed=4), 1e-5, 1e-4)
+    _check(_run(exe, d, (1, 64, 2, 64), mode="fixed", seed=5), 1e-5, None)
