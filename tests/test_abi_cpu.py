@@ -338,20 +338,37 @@ amdhsa.target:   amdgcn-amd-amdhsa--gfx950
 
 
 class _FakeLib(object):
-    """Stands in for the loaded library: every entry point accepts anything and reports success.
-    `calls` lists the names looked up, in order."""
+    """Stands in for the loaded library: every entry point reports success without doing anything, after
+    checking the call against the header's prototype (argument count; a pointer where a pointer is declared,
+    an integer where an integer is).  `calls` lists the names looked up, in order."""
     calls = []
+    _protos = None
+
+    @classmethod
+    def _check(cls, name, args):
+        if cls._protos is None:
+            import test_abi_signatures_cpu as sig
+            cls._protos = sig._prototypes(open(os.path.join(ROOT, "include", "l1attn_hip.h")).read(), ";")
+        ret, params = cls._protos[name]
+        assert len(args) == len(params), "%s called with %d arguments, declared with %d" % (name, len(args), len(params))
+        for i, (a, p) in enumerate(zip(args, params)):
+            if p == "ptr":
+                ok = a is None or isinstance(a, (ctypes.c_void_p, ctypes.Array))
+            else:
+                ok = isinstance(a, int)
+            assert ok, "%s argument %d: %r where the header declares %s" % (name, i, a, p)
 
     def __getattr__(self, name):
         _FakeLib.calls.append(name)
-        if name.endswith("_bytes"):
-            return lambda *a: 256
-        if name == "l1attn_sparse_plan_check":
-            def chk(buf, E, T, hdr, st):
-                hdr[4], hdr[5] = 3, 2
-                return 0
-            return chk
-        return lambda *a: 0
+
+        def call(*a):
+            _FakeLib._check(name, a)
+            if name.endswith("_bytes"):
+                return 256
+            if name == "l1attn_sparse_plan_check":
+                a[3][4], a[3][5] = 3, 2
+            return 0
+        return call
 
 
 def test_driver_control_flow_without_a_gpu(monkeypatch):
@@ -387,6 +404,8 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
     assert drv.enable_experimental("rows16", "fused", "fixed") == frozenset(drv.EXPERIMENTAL)
     a, = drv.dense_forward(q, k)
     assert a.shape == (B, T, T, H)
+    a, = drv.dense_forward_fixed(q, k)
+    assert a.shape == (B, T, T, H) and _FakeLib.calls[-2:] == ["l1attn_dense_fwd_fixed_workspace_bytes", "l1attn_dense_fwd_fixed_f32"]
     dq, dk = drv.dense_backward(torch.zeros(B, T, T, H), q, k)
     assert dq.shape == q.shape and dk.shape == k.shape
     with pytest.raises(RuntimeError, match="d_attn must be"):
