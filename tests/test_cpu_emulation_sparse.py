@@ -57,7 +57,7 @@ def _plan_arrays(co, T):
     return [i32(dp), i32(sp), i32(src[od]), i32(od), i32(dst[os_]), i32(slot_of_row[os_]), i32(long_d), i32(long_s)]
 
 
-def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind):
+def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind, extra_env=None):
     B, T, H, W = q.shape
     Wv, E = vf.shape[3], co.shape[0]
     arrays = _plan_arrays(co, T)
@@ -69,7 +69,7 @@ def _run(exe, tmp_path, vf, vb, q, k, co, sm, bidi, kind):
         dvo = torch.randn(B, T, H, Wv, generator=torch.Generator().manual_seed(77))
         for x in (vf, vb, q, k, dvo):
             f.write(x.float().contiguous().numpy().tobytes())
-    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0", **(extra_env or {}))
     r = subprocess.run([exe, fin, fout], env=env, capture_output=True, text=True)
     assert r.returncode == 0, (r.returncode, r.stderr[-2000:])
     raw = np.fromfile(fout, np.float64)
@@ -163,3 +163,29 @@ def test_sparse_forward_long_segment_on_cpu(runner, tmp_path):
     assert cf.rel_err(vob, cf.bidi_value(vf.double(), vb.double(), q.double(), k.double(), co, True)) <= 1e-5
     _check_grads(vf, vb, q, k, co, True, True, 1e-4)  # long segments in both backward passes
 
+
+
+def test_sparse_kernels_under_thread_sanitizer(tmp_path_factory):
+    """Forward and backward, one-directional and bidirectional, float32 and float16 rows, a hub in each direction
+    (long segments): the wave-level exchanges through LDS and the workgroup barriers of sparse.hip leave no data
+    race among the OS threads that stand for the lanes."""
+    d = tmp_path_factory.mktemp("emu_sparse_tsan")
+    exe = str(d / "run_sparse")
+    subprocess.run([CLANG, "-std=c++20", "-O1", "-gline-tables-only", "-pthread", "-fsanitize=thread", "-I", EMU, "-x", "c++",
+                    os.path.join(EMU, "run_sparse.cpp"), "-o", exe], check=True)
+    env = {"TSAN_OPTIONS": "halt_on_error=1 report_signal_unsafe=0"}
+    for (B, T, H, W, Wv, E, hub), kind, bidi in (((1, 24, 8, 32, 32, 150, False), "f32", True),
+                                                 ((1, 30, 4, 64, 64, 400, True), "f32", False),
+                                                 ((1, 30, 4, 64, 64, 400, True), "f16", True),
+                                                 ((1, 20, 3, 8, 12, 90, False), "bf16", False)):
+        g = torch.Generator().manual_seed(E)
+        co = torch.randint(0, T, (E, 2), generator=g)
+        if hub:
+            co[:160, 0], co[160:300, 1] = 3, 5
+        dt = TORCH_T.get(kind, torch.float32)
+        q, k = (torch.randn(B, T, H, W, generator=g).to(dt).float() for _ in range(2))
+        vf, vb = (torch.randn(B, T, H, Wv, generator=g).to(dt).float() for _ in range(2))
+        vo, _, _ = _run(exe, d, vf, vb, q, k, co, True, bidi, kind, extra_env=env)
+        x = [t.double() for t in (vf, vb, q, k)]
+        ref = cf.bidi_value(*x, co, True) if bidi else cf.sparse_value(x[0], x[2], x[3], co, True)
+        assert cf.rel_err(vo, ref) <= (1e-5 if kind == "f32" else TOL[kind])
