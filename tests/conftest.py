@@ -28,23 +28,28 @@ EMU = os.path.join(ROOT, "tests", "cpu_emu")
 CLANG = "/opt/rocm/llvm/bin/clang++"
 
 
-RUNNERS = {"fused": "g++", "sparse": CLANG, "ranks": "g++", "dense": "g++"}
+# runner -> (source name, host compiler, sanitizers)
+RUNNERS = {"fused": ("fused", "g++", "address,undefined"), "sparse": ("sparse", CLANG, "address,undefined"),
+           "ranks": ("ranks", "g++", "address,undefined"), "dense": ("dense", "g++", "address,undefined"),
+           "fused_tsan": ("fused", "g++", "thread"), "sparse_tsan": ("sparse", CLANG, "thread"),
+           "dense_tsan": ("dense", "g++", "thread")}
 
 
 @pytest.fixture(scope="session")
 def _emu_builds(tmp_path_factory):
-    """The CPU builds of the kernel files' runners (tests/cpu_emu/run_<name>.cpp) under AddressSanitizer and
-    UndefinedBehaviorSanitizer, started side by side at the first request and shared by every emulation test
-    module of the session.  Line tables only: enough for a sanitizer report to name the line."""
+    """The CPU builds of the kernel files' runners (tests/cpu_emu/run_<name>.cpp), under AddressSanitizer +
+    UndefinedBehaviorSanitizer and under ThreadSanitizer, started side by side at the first request and shared by
+    every emulation test module of the session.  Line tables only: enough for a sanitizer report to name the line."""
     d = tmp_path_factory.mktemp("emu")
     jobs = {}
-    for name, cxx in RUNNERS.items():
+    for name, (src, cxx, san) in RUNNERS.items():
         if cxx == CLANG and not os.path.exists(CLANG):
             continue
         exe = str(d / ("run_" + name))
         lines = "-gline-tables-only" if cxx == CLANG else "-g1"
-        cmd = [cxx, "-std=c++20", "-O1", lines, "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
-               "-I", EMU, "-x", "c++", os.path.join(EMU, "run_%s.cpp" % name), "-o", exe]
+        cmd = [cxx, "-std=c++20", "-O1", lines, "-pthread", "-fsanitize=" + san] + \
+              (["-fno-sanitize-recover=all"] if san != "thread" else []) + \
+              ["-I", EMU, "-x", "c++", os.path.join(EMU, "run_%s.cpp" % src), "-o", exe]
         jobs[name] = (exe, cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
     return jobs
 
@@ -76,3 +81,18 @@ def emu_ranks(_emu_builds):
 @pytest.fixture(scope="session")
 def emu_dense(_emu_builds):
     return _emu_runner(_emu_builds, "dense")
+
+
+@pytest.fixture(scope="session")
+def emu_fused_tsan(_emu_builds):
+    return _emu_runner(_emu_builds, "fused_tsan")
+
+
+@pytest.fixture(scope="session")
+def emu_sparse_tsan(_emu_builds):
+    return _emu_runner(_emu_builds, "sparse_tsan")
+
+
+@pytest.fixture(scope="session")
+def emu_dense_tsan(_emu_builds):
+    return _emu_runner(_emu_builds, "dense_tsan")

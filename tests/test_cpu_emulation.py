@@ -29,12 +29,8 @@ def runner(emu_fused):
 
 
 @pytest.fixture(scope="module")
-def runner_tsan(tmp_path_factory):
-    exe = str(tmp_path_factory.mktemp("emu_tsan") / "run_fused")
-    cmd = ["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=thread", "-I", EMU, "-x", "c++",
-           os.path.join(EMU, "run_fused.cpp"), "-o", exe]
-    subprocess.run(cmd, check=True)
-    return exe
+def runner_tsan(emu_fused_tsan):
+    return emu_fused_tsan
 
 
 def _run(exe, tmp_path, q, k, v, misalign=0, pipe=False):

@@ -157,14 +157,11 @@ def test_fixed_point_forward_kernel(runner, tmp_path, shape):
     _check(_run(runner, tmp_path, shape, mode="fixed", seed=sum(shape)), 1e-5, None)
 
 
-def test_dense_kernels_under_thread_sanitizer(tmp_path_factory):
+def test_dense_kernels_under_thread_sanitizer(tmp_path, emu_dense_tsan):
     """A barrier missing between a step's LDS writes and reads, or between two steps, is a data race here.
     Shapes with whole column chunks only: lanes beyond the last column deliberately redo the chunk's first
     column and store the same bits to the same address, which ThreadSanitizer rightly calls a race."""
-    d = tmp_path_factory.mktemp("emu_dense_tsan")
-    exe = str(d / "run_dense")
-    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-pthread", "-fsanitize=thread", "-I", EMU, "-x", "c++",
-                    os.path.join(EMU, "run_dense.cpp"), "-o", exe], check=True)
+    d, exe = tmp_path, emu_dense_tsan
     _check(_run(exe, d, (1, 64, 4, 32), seed=1), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 70, 3, 64), seed=2), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 128, 4, 64), extra=("wide", 64, 1, 2), seed=3), 1e-5, 1e-4)

@@ -165,14 +165,11 @@ def test_sparse_forward_long_segment_on_cpu(runner, tmp_path):
 
 
 
-def test_sparse_kernels_under_thread_sanitizer(tmp_path_factory):
+def test_sparse_kernels_under_thread_sanitizer(tmp_path, emu_sparse_tsan):
     """Forward and backward, one-directional and bidirectional, float32 and float16 rows, a hub in each direction
     (long segments): the wave-level exchanges through LDS and the workgroup barriers of sparse.hip leave no data
     race among the OS threads that stand for the lanes."""
-    d = tmp_path_factory.mktemp("emu_sparse_tsan")
-    exe = str(d / "run_sparse")
-    subprocess.run([CLANG, "-std=c++20", "-O1", "-gline-tables-only", "-pthread", "-fsanitize=thread", "-I", EMU, "-x", "c++",
-                    os.path.join(EMU, "run_sparse.cpp"), "-o", exe], check=True)
+    d, exe = tmp_path, emu_sparse_tsan
     env = {"TSAN_OPTIONS": "halt_on_error=1 report_signal_unsafe=0"}
     for (B, T, H, W, Wv, E, hub), kind, bidi in (((1, 24, 8, 32, 32, 150, False), "f32", True),
                                                  ((1, 30, 4, 64, 64, 400, True), "f32", False),
