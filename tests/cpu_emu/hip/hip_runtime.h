@@ -12,6 +12,7 @@
 #pragma once
 #include <math.h>
 #include <stddef.h>
+#include <stdio.h>
 #include <stdint.h>
 #include <algorithm>
 #include <barrier>
@@ -58,6 +59,10 @@ inline std::unique_ptr<std::barrier<>> wg_barrier;  // the running workgroup's _
 // bracketed by a barrier among the wave's 64 threads.
 inline std::vector<std::unique_ptr<std::barrier<>>> wave_barrier;
 inline std::vector<double> wave_slots;  // 64 exchange slots per wave
+// A runner may ask to see every launch (kernel expression as written at the launch site, grid, block, dynamic LDS
+// bytes) and may set `dry`: the launch is then reported and checked against the limits of a HIP launch, not run.
+inline void (*on_launch)(const char* kernel, dim3 grid, dim3 block, size_t lds) = nullptr;
+inline bool dry = false;
 inline unsigned char* dynamic_lds = nullptr;  // the launch's dynamically sized LDS array, exactly `lds` bytes
 inline unsigned flat_tid() { return threadIdx_.x + blockDim_.x * (threadIdx_.y + blockDim_.y * threadIdx_.z); }
 inline void wave_sync() { wave_barrier[flat_tid() >> 6]->arrive_and_wait(); }
@@ -135,8 +140,18 @@ static inline void emu_buf_fadd(float x, __amdgpu_buffer_rsrc_t r, int v, int s)
 static inline void __syncthreads() { emu::wg_barrier->arrive_and_wait(); }
 
 template <typename K, typename... A>
-static inline void emu_launch(K kernel, dim3 grid, dim3 block, size_t lds, A... args)
+static inline void emu_launch(const char* name, K kernel, dim3 grid, dim3 block, size_t lds, A... args)
 {
+	// what hipLaunchKernelGGL would refuse (the library reads the error after every launch; here it is fatal)
+	const uint64_t nthreads = (uint64_t)block.x * block.y * block.z;
+	if (!(grid.x >= 1 && grid.y >= 1 && grid.z >= 1 && grid.x <= 2147483647u && grid.y <= 65535u && grid.z <= 65535u &&
+	      nthreads >= 1 && nthreads <= 1024 && lds <= 64 * 1024)) {
+		fprintf(stderr, "invalid launch of %s: grid %u %u %u block %u %u %u lds %zu\n", name, grid.x, grid.y, grid.z, block.x,
+		        block.y, block.z, lds);
+		abort();
+	}
+	if (emu::on_launch) emu::on_launch(name, grid, block, lds);
+	if (emu::dry) return;
 	// exactly sized, so that AddressSanitizer sees an access beyond the launch's LDS size
 	std::unique_ptr<unsigned char[]> lds_mem(lds ? new unsigned char[lds] : nullptr);
 	emu::dynamic_lds = lds_mem.get();
@@ -167,4 +182,4 @@ static inline void emu_launch(K kernel, dim3 grid, dim3 block, size_t lds, A... 
 	emu::n_threads_run += (long)nt * nblocks;
 }
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
-	emu_launch(kernel, dim3(grid), dim3(block), (size_t)(lds), __VA_ARGS__)
+	emu_launch(#kernel, kernel, dim3(grid), dim3(block), (size_t)(lds), __VA_ARGS__)

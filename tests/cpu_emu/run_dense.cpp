@@ -2,6 +2,9 @@
 // for the host with the stand-in headers next to this file, through the library's own entry points: the host
 // logic that picks kernels, grids and workspace is the library's, unchanged.
 //   run_dense <in> <out> <f32|f64|fixed> [wide <tt_rows> <rank 0|1> <group>]
+//   run_dense dims <B> <T> <H> <W>      launch geometry only, at any size: every launch the float32 forward,
+//                                       backward and fixed-point forward would make is checked against the limits
+//                                       of a HIP launch and printed (kernel, grid, block, LDS bytes); nothing runs
 // in : int64 B,T,H,W then q,k [B,T,H,W] and dA [B,T,T,H] in the chosen type (fixed: float32)
 // out: attn [B,T,T,H], dq, dk [B,T,H,W] (fixed: attn only), then int64[16] of l1attn_dense_bwd_plan_info
 // Every buffer is malloc'ed at its exact size and every output starts as NaN, so AddressSanitizer reports an
@@ -62,6 +65,7 @@ int l1_launch_column_ranks(const float* q, const float* k, float* rq, float* rk,
                            int64_t W, hipStream_t)
 {
 	if (!l1_column_ranks_ok(B, T, H, W)) return L1ATTN_ERR_RANGE;
+	if (emu::dry) return L1ATTN_OK;
 	const int64_t HW = H * W;
 	std::vector<float> col((size_t)T);
 	for (int64_t b = 0; b < B; b++)
@@ -221,8 +225,33 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, const char* mode, int argc,
 	return 0;
 }
 
+static void print_launch(const char* kernel, dim3 g, dim3 b, size_t lds)
+{
+	printf("%s | %u %u %u | %u | %zu\n", kernel, g.x, g.y, g.z, b.x * b.y * b.z, lds);
+}
+
+// no memory behind the pointers: the host logic only looks at their alignment
+static int dims(int64_t B, int64_t T, int64_t H, int64_t W)
+{
+	emu::dry = true;
+	emu::on_launch = print_launch;
+	float* const p = (float*)(uintptr_t)0x100000;
+	const size_t wf = l1attn_dense_fwd_workspace_bytes(B, T, H, W), wb = l1attn_dense_bwd_workspace_bytes(B, T, H, W);
+	printf("forward workspace %zu\n", wf);
+	int rc = l1attn_dense_fwd_ws_f32(p, p, p, B, T, H, W, wf ? p : nullptr, wf, nullptr);
+	printf("forward rc %d\nbackward workspace %zu\n", rc, wb);
+	rc = l1attn_dense_bwd_f32(p, p, p, p, p, B, T, H, W, wb ? p : nullptr, wb, nullptr);
+	printf("backward rc %d\n", rc);
+	if ((W == 32 || W == 64) && T >= 32) {
+		rc = l1attn_dense_fwd_fixed_f32(p, p, p, B, T, H, W, p, l1attn_dense_fwd_fixed_workspace_bytes(B, T, H, W), nullptr);
+		printf("fixed rc %d\n", rc);
+	}
+	return 0;
+}
+
 int main(int argc, char** argv)
 {
+	if (argc == 6 && !strcmp(argv[1], "dims")) return dims(atoll(argv[2]), atoll(argv[3]), atoll(argv[4]), atoll(argv[5]));
 	if (argc < 4) return 2;
 	FILE* fi = fopen(argv[1], "rb");
 	FILE* fo = fopen(argv[2], "wb");

@@ -13,6 +13,7 @@ barrier is a data race).  This says nothing about timing, register allocation or
 The 512-thread tile kernels are chosen by the library from 1024 tokens and a few thousand workgroups on; the runner
 can build their plan for any length ("wide"), which is how they are walked here at 100 to 260 tokens."""
 import os
+import re
 import struct
 import subprocess
 
@@ -167,3 +168,42 @@ def test_dense_kernels_under_thread_sanitizer(tmp_path, emu_dense_tsan):
     _check(_run(exe, d, (1, 128, 4, 64), extra=("wide", 64, 1, 2), seed=3), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 136, 2, 64), extra=("wide", 72, 0, 1), seed=4), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 64, 2, 64), mode="fixed", seed=5), 1e-5, None)
+
+
+def _dims(exe, shape):
+    r = subprocess.run([exe, "dims"] + [str(x) for x in shape], env=ENV, capture_output=True, text=True)
+    assert r.returncode == 0, (shape, r.stderr[-800:])   # an invalid launch aborts the runner
+    rcs = dict(re.findall(r"^(forward|backward|fixed) rc (-?\d+)$", r.stdout, flags=re.M))
+    launches = [(m[0].strip("()"), tuple(int(x) for x in m[1].split()), int(m[2]), int(m[3]))
+                for m in re.findall(r"^(.+?) \| (\d+ \d+ \d+) \| (\d+) \| (\d+)$", r.stdout, flags=re.M)]
+    return rcs, launches
+
+
+def test_launch_geometry_at_full_size(runner):
+    """Every launch of the dense forward, backward and fixed-point forward at sizes no emulation can run: the
+    three dense baseline configurations and the 40 cells of the reference's timing grid at its batch of 512
+    (benchmark.py:57-66).  The host logic runs as in the library with nothing behind the pointers; the runner
+    checks each launch against what a HIP launch accepts (grid 2^31-1 x 65535 x 65535, 1024 threads, 64 KiB of
+    dynamic LDS) and reports it."""
+    rcs, launches = _dims(runner, (8, 4096, 16, 64))
+    assert rcs == {"forward": "0", "backward": "0", "fixed": "0"}
+    assert launches[:4] == [("dense_fwd_f32_pipe<64, false>", (64, 4, 8), 1024, 0),
+                            ("dense_bwd_f32_fast<64, 512, 4, true, true, true>", (16, 2, 8), 512, 4 * 8 * 68 * 4),
+                            ("dense_bwd_reduce_colsum", (2048, 1, 1), 256, 0),
+                            ("dense_bwd_reduce_dk<true, true>", (32768, 1, 1), 256, 0)]
+    rcs, launches = _dims(runner, (16, 1024, 8, 64))
+    assert rcs["backward"] == "0" and launches[1] == ("dense_bwd_f32_fast<64, 512, 4, false, false, true>", (16, 1, 16), 512, 8704)
+    assert _dims(runner, (2, 64, 4, 32))[0]["backward"] == "0"
+    kernels = set()
+    for T in (16, 32, 64, 128, 256):
+        for W in (16, 32, 33, 64, 65, 96, 97, 128):
+            rcs, launches = _dims(runner, (512, T, 8, W))
+            assert rcs["forward"] == "0" and rcs["backward"] == "0", (T, W, rcs)
+            kernels.update(name for name, _, _, _ in launches)
+    # the grid walks the one-workgroup forward, five widths of the tiled forward and the 32-token backward tiles
+    assert {"dense_fwd_small<T>", "dense_fwd_f32_fast<16>", "dense_fwd_f32_pipe<32, false>", "dense_fwd_f32_fast<48>",
+            "dense_fwd_f32_pipe<64, false>", "dense_fwd_f32_fast<80>", "dense_fwd_f32_pipe<96, false>", "dense_pad_rows",
+            "dense_bwd_f32_fast<32, 1024, 1, false, false, false>"} <= kernels
+    # sizes at the edges of what the host logic accepts end in a return code, not in a launch that HIP would refuse
+    for shape in ((65535, 32, 1, 32), (70000, 32, 1, 32), (1, 8192, 64, 128), (1, 100000, 1, 32), (3, 16, 4096, 16)):
+        _dims(runner, shape)
