@@ -394,7 +394,7 @@ __device__ __forceinline__ float row16_sum_to_last(float x)
 // TT values and store the column sum to csp [n_ttiles][nb][T][H] (the reduction kernel needs it),
 // and every thread keeps the running sum over src rows of up to NR (head, dst token) slots (the
 // row sums that dq needs after the loop).  dkp then holds the raw sum(hv*g) partials.
-template <int TT, int MAXTHREADS, int PER, bool RANK, bool GROUPED, bool FAST>
+template <int TT, int MAXTHREADS, int PER, bool RANK, bool GROUPED, bool FAST, bool DEEP = false>
 __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __restrict__ dA,
                                                                    const float* __restrict__ q,
                                                                    const float* __restrict__ k,
@@ -515,6 +515,136 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) asm volatile("" : "+v"(k_pre[j]));
 	};
+	if constexpr (DEEP) {
+	// Two steps of prefetch distance.  With one (below), the wait at the end of a step is for the youngest
+	// vector-memory operations of the wave, i.e. for everything: the loads of the next step's values and, older
+	// than those, the dk stores of the step before and the column-sum store of this one.  Here two register sets
+	// alternate: the set a step has just put into LDS is refilled with the values of the step after next, and
+	// the wait at the end of the step is for the other set, whose loads are a whole step old; the stores issued
+	// since (this step's column sums, the previous step's dk rows) and the refill stay in flight across it.
+	// The step loop runs two steps per iteration, so that the sets are fixed registers.
+	static_assert(!DEEP || FAST, "two-step prefetch: branch-free form only");
+	float g_a[PER], k_a[BWD_SJ], g_b[PER], k_b[BWD_SJ];
+	auto fetch = [&](float (&g)[PER], float (&kk)[BWD_SJ]) {
+		const buf_t rd = make_buf(dA_pf), rk = make_buf(k_pf);
+#pragma unroll
+		for (int r = 0; r < PER; r++) g[r] = buf_load(rd, st_off[0] * 4u, (unsigned)r * dA_row_bytes);
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) kk[j] = buf_load(rk, col_bytes, (unsigned)j * row_bytes);
+	};
+	auto arrived = [&](float (&g)[PER], float (&kk)[BWD_SJ]) {
+#pragma unroll
+		for (int r = 0; r < PER; r++) asm volatile("" : "+v"(g[r]));
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) asm volatile("" : "+v"(kk[j]));
+	};
+	// one step: g_use / k_use hold its values (arrived); g_nxt / k_nxt are in flight for the step after it
+	auto step = [&](const int s0, float (&g_use)[PER], float (&k_use)[BWD_SJ], float (&g_nxt)[PER], float (&k_nxt)[BWD_SJ]) {
+		lds_barrier();  // the previous step's LDS reads are done
+#pragma unroll
+		for (int r = 0; r < PER; r++) gl[st_lds[0] + r * HB * TTP] = g_use[r];
+		float kc[BWD_SJ], dka[BWD_SJ];
+#pragma unroll
+		for (int j = 0; j < BWD_SJ; j++) {
+			kc[j] = RANK ? k_use[j] : k_use[j] * BWD_PRESCALE;
+			dka[j] = 0.0f;
+		}
+		lds_barrier();
+		// the step after next into the set just consumed; the last two steps read rows they have read before
+		const bool more = s0 + 2 * BWD_SJ < Tn;
+		dA_pf += more ? dA_step : 0;
+		k_pf += more ? k_step : 0;
+		fetch(g_use, k_use);
+		const buf_t rp = make_buf(dkp_cur);
+		{
+			// All dA values of this step for the lane's head, each float4 read D blocks ahead of its use, one read
+			// between two blocks of math.  Every instruction of a wave takes an issue slot, an s_waitcnt too: the
+			// branch-free form waits once per BL blocks instead of once per block (LDS reads return in order, so
+			// blocks bi..bi+BL-1 are there once no more than the D-BL+1 reads issued after them are outstanding).
+			const float4* gp0 = reinterpret_cast<const float4*>(gl + hl * TTP);
+			constexpr int NI4 = TT / 4, NBLK = BWD_SJ * NI4, BL = FAST ? BWD_LDS_BATCH : 1, D = 2 * BL - 1, RING = D + 1;
+			auto g_at = [&](int bi) { return gp0[((bi / NI4) * HB * TTP) / 4 + bi % NI4]; };
+			float4 g_ring[RING];
+#pragma unroll
+			for (int d = 0; d < D; d++) g_ring[d] = g_at(d);
+			// RANK: the tile values for the sums are read here and added up after the first src row's math,
+			// by which time they have arrived.  Column sums: row = jj*HB + hh of the tile, sixteen lanes per
+			// row (the host checks BWD_SJ*HB*16 <= blockDim.x).  Row sums: this thread's (head, dst token) slots.
+			constexpr int NM = (TT / 4 + 15) / 16;
+			const int cs_sub = threadIdx.x & 15, cs_row = threadIdx.x >> 4;
+			float4 cs_v[NM];
+			float rs_v[NR][BWD_SJ];
+			if (RANK) {
+				const float4* rp = reinterpret_cast<const float4*>(gl + cs_row * TTP);
+#pragma unroll
+				for (int m = 0; m < NM; m++) {
+					cs_v[m] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+					// FAST (64-token tiles, 64*HB threads): every group of sixteen lanes has a row, every lane a float4
+					if (FAST || (cs_row < BWD_SJ * HB && cs_sub + 16 * m < TT / 4)) cs_v[m] = rp[cs_sub + 16 * m];
+				}
+#pragma unroll
+				for (int n = 0; n < NR; n++) {
+#pragma unroll
+					for (int jj = 0; jj < BWD_SJ; jj++) rs_v[n][jj] = (FAST || rs_lds[n] >= 0) ? gl[jj * HB * TTP + rs_lds[n]] : 0.0f;
+				}
+			}
+#pragma unroll
+			for (int bi = 0; bi < NBLK; bi++) {
+				{
+					const int j = bi / NI4, i4 = bi % NI4;
+					if (bi + D < NBLK) g_ring[(bi + D) % RING] = g_at(bi + D);
+					if (BL > 1 && bi > 0 && bi % BL == 0) {
+						// s_waitcnt immediate: vmcnt and expcnt at their maxima, lgkmcnt in bits 11:8
+						if (bi + BL < NBLK) __builtin_amdgcn_s_waitcnt(0xC07F | ((D - BL + 1) << 8));
+						else __builtin_amdgcn_s_waitcnt(0xC07F);
+					}
+					__builtin_amdgcn_sched_barrier(0);
+					if (RANK && j == 1 && i4 == 0) {
+						// keep the loaded values opaque up to here, or the adds (and the wait for the loads)
+						// are hoisted in front of the first src row's math
+#pragma unroll
+						for (int m = 0; m < NM; m++)
+							asm volatile("" : "+v"(cs_v[m].x), "+v"(cs_v[m].y), "+v"(cs_v[m].z), "+v"(cs_v[m].w));
+#pragma unroll
+						for (int n = 0; n < NR; n++) {
+#pragma unroll
+							for (int jj = 0; jj < BWD_SJ; jj++) asm volatile("" : "+v"(rs_v[n][jj]));
+						}
+						float a = 0.0f;
+#pragma unroll
+						for (int m = 0; m < NM; m++) a += (cs_v[m].x + cs_v[m].y) + (cs_v[m].z + cs_v[m].w);
+						a = row16_sum_to_last(a);
+						const int jj = cs_row / HB, s = s0 + jj;
+						if (cs_sub == 15 && (FAST || (cs_row < BWD_SJ * HB && s < Tn))) csp_b[(int64_t)s * H + (cs_row - jj * HB)] = a;
+#pragma unroll
+						for (int n = 0; n < NR; n++) rs_acc[n] += (rs_v[n][0] + rs_v[n][1]) + (rs_v[n][2] + rs_v[n][3]);
+						__builtin_amdgcn_sched_barrier(0);
+					}
+					if (RANK) pair_step4_rank(&qc[i4 * 4], kc[j], g_ring[bi % RING], &dqa[i4 * 4], dka[j]);
+					else pair_step4(&qc[i4 * 4], kc[j], g_ring[bi % RING], &dqa[i4 * 4], dka[j]);
+				}
+			}
+		}
+		arrived(g_nxt, k_nxt);
+		if (!GROUPED || u == 0) {
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) buf_store(RANK ? dka[j] : dka[j] * scale, rp, col_bytes, (unsigned)j * row_bytes);
+		} else {
+#pragma unroll
+			for (int j = 0; j < BWD_SJ; j++) buf_add(RANK ? dka[j] : dka[j] * scale, rp, col_bytes, (unsigned)j * row_bytes);
+		}
+		dkp_cur += (int64_t)BWD_SJ * HW;
+	};
+	fetch(g_a, k_a);  // step 0
+	dA_pf += BWD_SJ < Tn ? dA_step : 0;
+	k_pf += BWD_SJ < Tn ? k_step : 0;
+	fetch(g_b, k_b);  // step 1
+	arrived(g_a, k_a);
+	for (int s0 = 0; s0 < Tn; s0 += 2 * BWD_SJ) {  // (the host picks this form only for T a multiple of 2*BWD_SJ)
+		step(s0, g_a, k_a, g_b, k_b);
+		step(s0 + BWD_SJ, g_b, k_b, g_a, k_a);
+	}
+	} else {
 	prefetch(0);
 	settle();
 
@@ -649,6 +779,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 			if (FAST || s < Tn) (dkp_b + (int64_t)s * HW)[col] = GROUPED ? dk_old[j] + v : v;
 		}
 	}
+	}  // one or two steps of prefetch distance
 	float* const dq_b = dq + (int64_t)b * Tn * HW;
 	if (RANK) {
 		lds_barrier();  // the last step's tile reads are done
@@ -863,6 +994,7 @@ struct BwdPlan {
 	bool rank;        // three-instruction pair-elements on column ranks
 	int threads, n_cc, n_tt, tt_rows, per;
 	bool branch_free;        // every workgroup of the launch runs whole tiles and whole steps
+	bool deep;               // branch-free form with two steps of prefetch distance (on request, see below)
 	int group, n_groups;     // consecutive dst tiles per workgroup (sharing one dk partial); workgroups along T
 	size_t lds_bytes;
 	size_t partial_bytes;    // partial-dk scratch for one batch (0 when a single dst tile)
@@ -882,6 +1014,18 @@ bool l1_rank_sort_is_merge()
 		return e && e[0] == 'm';
 	}();
 	return merge;
+}
+
+// Prefetch distance of the branch-free step loop: one step (the default: it is the one that has run the GPU
+// tests) or two when the environment holds L1ATTN_BWD_PREFETCH=2.  Same sums in the same order either way, so
+// the results are bit-identical; the choice is read once.
+bool l1_bwd_prefetch_is_deep()
+{
+	static const bool deep = [] {
+		const char* e = getenv("L1ATTN_BWD_PREFETCH");
+		return e && e[0] == '2';
+	}();
+	return deep;
 }
 
 BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
@@ -945,6 +1089,7 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.branch_free = p.wide && p.tt_rows == 64 && T % 64 == 0 && T % BWD_SJ == 0 && HW % p.threads == 0 &&
 	                (BWD_SJ * T + 128) * H < ((int64_t)1 << 29) &&
 	                p.threads % W == 0 && (int64_t)BWD_SJ * 64 * (p.threads / W) == (int64_t)4 * p.threads;
+	p.deep = p.branch_free && T % (2 * BWD_SJ) == 0 && l1_bwd_prefetch_is_deep();
 	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_groups * T * HW * sizeof(float) : 0;
 	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
 	p.rank_bytes = p.rank ? ((size_t)2 * T * HW + (size_t)(p.n_tt + 1) * T * H) * sizeof(float) : 0;
@@ -959,7 +1104,15 @@ void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* d
 	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV, RANKV, GRPV, FASTV>), grid, dim3(p.threads), p.lds_bytes, \
 	                   st, dA, q, k, dq, dkp, csp, T, H, W, scale, p.group)
 #define L1_BWD_CASE(TTV, MT, PERV, RANKV, GRPV) L1_BWD_CASE6(TTV, MT, PERV, RANKV, GRPV, false)
-	if (p.wide && p.branch_free) {
+#define L1_BWD_CASE_DEEP(RANKV, GRPV)                                                                         \
+	hipLaunchKernelGGL((dense_bwd_f32_fast<64, 512, 4, RANKV, GRPV, true, true>), grid, dim3(p.threads), p.lds_bytes, \
+	                   st, dA, q, k, dq, dkp, csp, T, H, W, scale, p.group)
+	if (p.wide && p.branch_free && p.deep) {
+		if (p.rank && p.group > 1) L1_BWD_CASE_DEEP(true, true);
+		else if (p.rank) L1_BWD_CASE_DEEP(true, false);
+		else if (p.group > 1) L1_BWD_CASE_DEEP(false, true);
+		else L1_BWD_CASE_DEEP(false, false);
+	} else if (p.wide && p.branch_free) {
 		// bwd_plan() sets branch_free only for 64-token tiles with four staged values per thread
 		if (p.rank && p.group > 1) L1_BWD_CASE6(64, 512, 4, true, true, true);
 		else if (p.rank) L1_BWD_CASE6(64, 512, 4, true, false, true);
@@ -993,6 +1146,7 @@ void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* d
 	}
 #undef L1_BWD_CASE
 #undef L1_BWD_CASE6
+#undef L1_BWD_CASE_DEEP
 }
 
 }  // namespace
@@ -1117,6 +1271,7 @@ int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64
 	info[8] = p.per; info[9] = p.group; info[10] = p.n_groups; info[11] = (int64_t)p.lds_bytes;
 	info[12] = (int64_t)p.per_batch_bytes;
 	info[13] = p.per_batch_bytes ? std::min<int64_t>(B, l1_cdiv(1024, (int64_t)p.n_groups * p.n_cc)) : B;
+	info[14] = p.deep;
 	return L1ATTN_OK;
 }
 

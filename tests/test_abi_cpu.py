@@ -3,6 +3,8 @@ declares, and its host-side argument logic (no kernel launch) behaves as documen
 import ctypes
 import os
 import re
+import subprocess
+import sys
 
 import pytest
 
@@ -77,7 +79,7 @@ def _plan(lib, B, T, H, W):
     a = (ctypes.c_int64 * 16)()
     assert lib.l1attn_dense_bwd_plan_info(B, T, H, W, a) == 0
     keys = ("tiled", "wide", "rank", "branch_free", "threads", "n_cc", "n_tt", "tt_rows", "per", "group", "n_groups",
-            "lds_bytes", "per_batch_bytes", "batches_per_launch")
+            "lds_bytes", "per_batch_bytes", "batches_per_launch", "deep")
     return dict(zip(keys, list(a)))
 
 
@@ -92,6 +94,7 @@ def test_dense_backward_plan_of_the_baseline_configurations(lib):
     assert c3["wide"] and c3["rank"] and c3["branch_free"]
     assert (c3["threads"], c3["n_cc"], c3["tt_rows"], c3["n_tt"], c3["group"], c3["n_groups"]) == (512, 2, 64, 64, 4, 16)
     assert c3["batches_per_launch"] == 8 and c3["per"] == 4 and c3["lds_bytes"] == 4 * 8 * 68 * 4
+    assert not (c1["deep"] or c2["deep"] or c3["deep"])                     # one step of prefetch distance unless asked
     # untiled shapes and empty problems
     assert not _plan(lib, 2, 3, 16, 7)["tiled"]
     assert _plan(lib, 0, 64, 4, 32) == {k: 0 for k in c1}
@@ -581,3 +584,24 @@ _Z4kernv: ; @k
         build.check_hot_loops(listing, (("kernv", 8, 2, 1.9),))
     with pytest.raises(RuntimeError, match="no loop"):
         build.check_hot_loops(listing, (("kernv", 16, 2, 4.0),))
+
+
+def test_backward_variants_are_chosen_by_the_environment_only(lib):
+    """L1ATTN_BWD_PREFETCH=2 turns the branch-free plans into their two-step-prefetch form and nothing else; it is
+    read once per process, hence the child process."""
+    code = ("import ctypes, sys; L = ctypes.CDLL(sys.argv[1]);"
+            "L.l1attn_dense_bwd_plan_info.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_void_p];"
+            "out = [];\n"
+            "for s in ((2, 64, 4, 32), (16, 1024, 8, 64), (8, 4096, 16, 64), (8, 4100, 16, 64), (2, 3, 16, 7)):\n"
+            "    a = (ctypes.c_int64 * 16)(); assert L.l1attn_dense_bwd_plan_info(*s, a) == 0; out.append(list(a))\n"
+            "print(out)")
+    import _l1attn_hip as drv
+    runs = {}
+    for depth in ("", "2"):
+        env = dict(os.environ, L1ATTN_BWD_PREFETCH=depth)
+        r = subprocess.run([sys.executable, "-c", code, drv._LIB_PATH], env=env, capture_output=True, text=True, check=True)
+        runs[depth] = eval(r.stdout)
+    for one, two in zip(runs[""], runs["2"]):
+        assert one[14] == 0 and two[14] == one[3]            # exactly the branch-free plans change
+        assert one[:14] == two[:14]                          # and in nothing but that flag
+    assert [p[14] for p in runs["2"]] == [0, 1, 1, 0, 0]

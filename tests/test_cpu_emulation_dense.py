@@ -143,12 +143,27 @@ def test_dense_backward_wide_tile_kernels(runner, tmp_path, shape, tt, rank, gro
     _check(_run(runner, tmp_path, shape, extra=("wide", tt, rank, group), seed=sum(shape) + tt, ties=ties), 1e-5, 1e-4)
 
 
+@pytest.mark.parametrize("shape,rank,group", [((2, 128, 2, 64), 0, 1), ((2, 128, 2, 64), 1, 1), ((3, 128, 4, 64), 0, 2),
+                                              ((1, 256, 4, 64), 1, 4), ((1, 64, 1, 64), 1, 1)])
+def test_two_step_prefetch_equals_the_one_step_loop(runner, tmp_path, shape, rank, group):
+    """dense_bwd_f32_fast<..., DEEP>: two register sets of prefetched values alternate and the step loop runs two
+    steps per iteration.  Same sums in the same order: dq and dk equal the one-step loop's bit for bit (and the
+    oracle's within the usual tolerance), also where the sequence is a single pair of steps short of nothing
+    (64 tokens = sixteen steps) and with half-integer inputs (ties)."""
+    deep = _run(runner, tmp_path, shape, extra=("wide", 64, rank, group, "deep"), seed=5, ties=bool(rank))
+    _check(deep, 1e-5, 1e-4)
+    one = _run(runner, tmp_path, shape, extra=("wide", 64, rank, group), seed=5, ties=bool(rank))
+    assert torch.equal(deep["dq"], one["dq"]) and torch.equal(deep["dk"], one["dk"])
+
+
 def test_plans_outside_the_kernels_limits_are_refused(runner, tmp_path):
     """The runner's plan builder mirrors the library's limits: sixteen lanes per staged (src row, head) in the rank
     form, at most eight staged values per thread."""
     for shape, extra in (((1, 100, 3, 33), ("wide", 72, 1, 1)), ((1, 150, 4, 32), ("wide", 88, 0, 1))):
         with pytest.raises(AssertionError, match=r"wide.*, 4, "):
             _run(runner, tmp_path, shape, extra=extra)
+    with pytest.raises(AssertionError, match=r"deep.*, 4, "):  # two-step prefetch exists in the branch-free form only
+        _run(runner, tmp_path, (1, 100, 2, 64), extra=("wide", 64, 0, 1, "deep"))
 
 
 @pytest.mark.parametrize("shape", [(1, 64, 4, 32), (1, 100, 3, 64), (2, 40, 2, 64)])
@@ -167,6 +182,8 @@ def test_dense_kernels_under_thread_sanitizer(tmp_path, emu_dense_tsan):
     _check(_run(exe, d, (1, 70, 3, 64), seed=2), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 128, 4, 64), extra=("wide", 64, 1, 2), seed=3), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 136, 2, 64), extra=("wide", 72, 0, 1), seed=4), 1e-5, 1e-4)
+    _check(_run(exe, d, (1, 128, 4, 64), extra=("wide", 64, 1, 2, "deep"), seed=6), 1e-5, 1e-4)
+    _check(_run(exe, d, (2, 64, 2, 64), extra=("wide", 64, 0, 1, "deep"), seed=7), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 64, 2, 64), mode="fixed", seed=5), 1e-5, None)
 
 

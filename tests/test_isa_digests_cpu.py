@@ -42,7 +42,12 @@ def _today(name):
     # the sparse kernels gained a storage type as last template argument; in the float32 and float64
     # instantiations it equals the compute type, which is how the tested kernels are named today
     m = re.match(r"(sparse\.hip sparse_\w+)<(float|double), (.*)>$", name)
-    return "%s<%s, %s, %s>" % (m.group(1), m.group(2), m.group(3), m.group(2)) if m else name
+    if m:
+        return "%s<%s, %s, %s>" % (m.group(1), m.group(2), m.group(3), m.group(2))
+    # the tiled dense backward gained a last template flag (two steps of prefetch distance); the tested kernels
+    # are the instantiations with the flag off
+    m = re.match(r"(dense\.hip dense_bwd_f32_fast)<(.*)>$", name)
+    return "%s<%s, false>" % (m.group(1), m.group(2)) if m else name
 
 
 def test_gpu_tested_kernels_are_unchanged():
