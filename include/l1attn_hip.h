@@ -91,8 +91,9 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
  *   8 staged d_attn values per thread, step   9 dst tiles per workgroup
  *  10 workgroups along T (= partial arrays)  11 LDS bytes per workgroup
  *  12 workspace bytes per batch              13 batches per launch with the full workspace
- *  14 step loop with two steps of prefetch distance (only with L1ATTN_BWD_PREFETCH=2 in the environment, read once
- *     per process: an alternative form of the branch-free loop with bit-identical results)
+ *  14 form of the branch-free step loop: 0, or with L1ATTN_BWD_PREFETCH=2 / =3 in the environment (read once per
+ *     process) 1 = two steps of prefetch distance, 2 = the same with two LDS planes and one barrier per step;
+ *     bit-identical results in all three
  *  15 reserved (0)
  * Returns 0, or a negative argument error.
  */

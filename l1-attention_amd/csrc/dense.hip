@@ -394,7 +394,7 @@ __device__ __forceinline__ float row16_sum_to_last(float x)
 // TT values and store the column sum to csp [n_ttiles][nb][T][H] (the reduction kernel needs it),
 // and every thread keeps the running sum over src rows of up to NR (head, dst token) slots (the
 // row sums that dq needs after the loop).  dkp then holds the raw sum(hv*g) partials.
-template <int TT, int MAXTHREADS, int PER, bool RANK, bool GROUPED, bool FAST, bool DEEP = false>
+template <int TT, int MAXTHREADS, int PER, bool RANK, bool GROUPED, bool FAST, int DEEP = 0>
 __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __restrict__ dA,
                                                                    const float* __restrict__ q,
                                                                    const float* __restrict__ k,
@@ -515,7 +515,7 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 #pragma unroll
 		for (int j = 0; j < BWD_SJ; j++) asm volatile("" : "+v"(k_pre[j]));
 	};
-	if constexpr (DEEP) {
+	if constexpr (DEEP != 0) {
 	// Two steps of prefetch distance.  With one (below), the wait at the end of a step is for the youngest
 	// vector-memory operations of the wave, i.e. for everything: the loads of the next step's values and, older
 	// than those, the dk stores of the step before and the column-sum store of this one.  Here two register sets
@@ -523,7 +523,11 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	// the wait at the end of the step is for the other set, whose loads are a whole step old; the stores issued
 	// since (this step's column sums, the previous step's dk rows) and the refill stay in flight across it.
 	// The step loop runs two steps per iteration, so that the sets are fixed registers.
-	static_assert(!DEEP || FAST, "two-step prefetch: branch-free form only");
+	// DEEP == 2: the two steps of an iteration also stage their tiles in two LDS planes (the host then gives the
+	// workgroup twice the LDS), and a step has one barrier instead of two.  The barrier that kept a step's LDS
+	// writes behind the previous step's reads is not needed: a thread writes plane p for step n+2 only after
+	// the barrier of step n+1, which every thread reaches after its reads of plane p in step n.
+	static_assert(DEEP == 0 || FAST, "two-step prefetch: branch-free form only");
 	float g_a[PER], k_a[BWD_SJ], g_b[PER], k_b[BWD_SJ];
 	auto fetch = [&](float (&g)[PER], float (&kk)[BWD_SJ]) {
 		const buf_t rd = make_buf(dA_pf), rk = make_buf(k_pf);
@@ -539,8 +543,11 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 		for (int j = 0; j < BWD_SJ; j++) asm volatile("" : "+v"(kk[j]));
 	};
 	// one step: g_use / k_use hold its values (arrived); g_nxt / k_nxt are in flight for the step after it
-	auto step = [&](const int s0, float (&g_use)[PER], float (&k_use)[BWD_SJ], float (&g_nxt)[PER], float (&k_nxt)[BWD_SJ]) {
-		lds_barrier();  // the previous step's LDS reads are done
+	float* const gl_planes = gl;
+	auto step = [&](const int s0, float (&g_use)[PER], float (&k_use)[BWD_SJ], float (&g_nxt)[PER], float (&k_nxt)[BWD_SJ],
+	                const int plane) {
+		float* const gl = gl_planes + plane * (BWD_SJ * HB * TTP);  // (hides the workgroup's array: this step's plane)
+		if (DEEP != 2) lds_barrier();  // the previous step's LDS reads are done
 #pragma unroll
 		for (int r = 0; r < PER; r++) gl[st_lds[0] + r * HB * TTP] = g_use[r];
 		float kc[BWD_SJ], dka[BWD_SJ];
@@ -640,9 +647,12 @@ __global__ __launch_bounds__(MAXTHREADS) void dense_bwd_f32_fast(const float* __
 	k_pf += BWD_SJ < Tn ? k_step : 0;
 	fetch(g_b, k_b);  // step 1
 	arrived(g_a, k_a);
+	// one barrier per dst tile where the steps have none before their LDS writes: the rank form's row sums of the
+	// workgroup's previous tile are read from plane 0 after its last barrier
+	if (DEEP == 2) lds_barrier();
 	for (int s0 = 0; s0 < Tn; s0 += 2 * BWD_SJ) {  // (the host picks this form only for T a multiple of 2*BWD_SJ)
-		step(s0, g_a, k_a, g_b, k_b);
-		step(s0 + BWD_SJ, g_b, k_b, g_a, k_a);
+		step(s0, g_a, k_a, g_b, k_b, 0);
+		step(s0 + BWD_SJ, g_b, k_b, g_a, k_a, DEEP == 2 ? 1 : 0);
 	}
 	} else {
 	prefetch(0);
@@ -994,7 +1004,7 @@ struct BwdPlan {
 	bool rank;        // three-instruction pair-elements on column ranks
 	int threads, n_cc, n_tt, tt_rows, per;
 	bool branch_free;        // every workgroup of the launch runs whole tiles and whole steps
-	bool deep;               // branch-free form with two steps of prefetch distance (on request, see below)
+	int deep;                // branch-free form with two steps of prefetch distance (1), and two LDS planes (2); on request
 	int group, n_groups;     // consecutive dst tiles per workgroup (sharing one dk partial); workgroups along T
 	size_t lds_bytes;
 	size_t partial_bytes;    // partial-dk scratch for one batch (0 when a single dst tile)
@@ -1016,16 +1026,17 @@ bool l1_rank_sort_is_merge()
 	return merge;
 }
 
-// Prefetch distance of the branch-free step loop: one step (the default: it is the one that has run the GPU
-// tests) or two when the environment holds L1ATTN_BWD_PREFETCH=2.  Same sums in the same order either way, so
-// the results are bit-identical; the choice is read once.
-bool l1_bwd_prefetch_is_deep()
+// Form of the branch-free step loop: one step of prefetch distance (the default: it is the one that has run the
+// GPU tests); two steps when the environment holds L1ATTN_BWD_PREFETCH=2; two steps, two LDS planes and one
+// barrier per step with L1ATTN_BWD_PREFETCH=3.  Same sums in the same order in all three, so the results are
+// bit-identical; the choice is read once.
+int l1_bwd_loop_form()
 {
-	static const bool deep = [] {
+	static const int form = [] {
 		const char* e = getenv("L1ATTN_BWD_PREFETCH");
-		return e && e[0] == '2';
+		return (e && e[0] == '2') ? 1 : (e && e[0] == '3') ? 2 : 0;
 	}();
-	return deep;
+	return form;
 }
 
 BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
@@ -1089,7 +1100,8 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.branch_free = p.wide && p.tt_rows == 64 && T % 64 == 0 && T % BWD_SJ == 0 && HW % p.threads == 0 &&
 	                (BWD_SJ * T + 128) * H < ((int64_t)1 << 29) &&
 	                p.threads % W == 0 && (int64_t)BWD_SJ * 64 * (p.threads / W) == (int64_t)4 * p.threads;
-	p.deep = p.branch_free && T % (2 * BWD_SJ) == 0 && l1_bwd_prefetch_is_deep();
+	p.deep = (p.branch_free && T % (2 * BWD_SJ) == 0) ? l1_bwd_loop_form() : 0;
+	if (p.deep == 2) p.lds_bytes *= 2;
 	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_groups * T * HW * sizeof(float) : 0;
 	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
 	p.rank_bytes = p.rank ? ((size_t)2 * T * HW + (size_t)(p.n_tt + 1) * T * H) * sizeof(float) : 0;
@@ -1104,14 +1116,19 @@ void launch_bwd_fast(const BwdPlan& p, dim3 grid, hipStream_t st, const float* d
 	hipLaunchKernelGGL((dense_bwd_f32_fast<TTV, MT, PERV, RANKV, GRPV, FASTV>), grid, dim3(p.threads), p.lds_bytes, \
 	                   st, dA, q, k, dq, dkp, csp, T, H, W, scale, p.group)
 #define L1_BWD_CASE(TTV, MT, PERV, RANKV, GRPV) L1_BWD_CASE6(TTV, MT, PERV, RANKV, GRPV, false)
-#define L1_BWD_CASE_DEEP(RANKV, GRPV)                                                                         \
-	hipLaunchKernelGGL((dense_bwd_f32_fast<64, 512, 4, RANKV, GRPV, true, true>), grid, dim3(p.threads), p.lds_bytes, \
+#define L1_BWD_CASE_DEEP(RANKV, GRPV, FORM)                                                                   \
+	hipLaunchKernelGGL((dense_bwd_f32_fast<64, 512, 4, RANKV, GRPV, true, FORM>), grid, dim3(p.threads), p.lds_bytes, \
 	                   st, dA, q, k, dq, dkp, csp, T, H, W, scale, p.group)
-	if (p.wide && p.branch_free && p.deep) {
-		if (p.rank && p.group > 1) L1_BWD_CASE_DEEP(true, true);
-		else if (p.rank) L1_BWD_CASE_DEEP(true, false);
-		else if (p.group > 1) L1_BWD_CASE_DEEP(false, true);
-		else L1_BWD_CASE_DEEP(false, false);
+	if (p.wide && p.branch_free && p.deep == 1) {
+		if (p.rank && p.group > 1) L1_BWD_CASE_DEEP(true, true, 1);
+		else if (p.rank) L1_BWD_CASE_DEEP(true, false, 1);
+		else if (p.group > 1) L1_BWD_CASE_DEEP(false, true, 1);
+		else L1_BWD_CASE_DEEP(false, false, 1);
+	} else if (p.wide && p.branch_free && p.deep == 2) {
+		if (p.rank && p.group > 1) L1_BWD_CASE_DEEP(true, true, 2);
+		else if (p.rank) L1_BWD_CASE_DEEP(true, false, 2);
+		else if (p.group > 1) L1_BWD_CASE_DEEP(false, true, 2);
+		else L1_BWD_CASE_DEEP(false, false, 2);
 	} else if (p.wide && p.branch_free) {
 		// bwd_plan() sets branch_free only for 64-token tiles with four staged values per thread
 		if (p.rank && p.group > 1) L1_BWD_CASE6(64, 512, 4, true, true, true);

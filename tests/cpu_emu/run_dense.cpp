@@ -1,7 +1,7 @@
 // TEST INFRASTRUCTURE: runs the dense operator of csrc/dense.hip (forward, backward, fixed-point forward), compiled
 // for the host with the stand-in headers next to this file, through the library's own entry points: the host
 // logic that picks kernels, grids and workspace is the library's, unchanged.
-//   run_dense <in> <out> <f32|f64|fixed> [wide <tt_rows> <rank 0|1> <group> [deep]]
+//   run_dense <in> <out> <f32|f64|fixed> [wide <tt_rows> <rank 0|1> <group> [deep|deep2]]
 //   run_dense dims <B> <T> <H> <W>      launch geometry only, at any size: every launch the float32 forward,
 //                                       backward and fixed-point forward would make is checked against the limits
 //                                       of a HIP launch and printed (kernel, grid, block, LDS bytes); nothing runs
@@ -91,7 +91,7 @@ int l1_launch_column_ranks_merge(const float* q, const float* k, float* rq, floa
 
 // The plan of the 512-thread tile kernels for any sequence length: bwd_plan()'s arithmetic with the tile height,
 // rank form and grouping given instead of chosen.  Returns fast = false where the kernels' own limits rule it out.
-static BwdPlan wide_plan(int64_t B, int64_t T, int64_t H, int64_t W, int tt_rows, bool rank, int group, bool deep)
+static BwdPlan wide_plan(int64_t B, int64_t T, int64_t H, int64_t W, int tt_rows, bool rank, int group, int deep)
 {
 	BwdPlan p{};
 	const int64_t HW = H * W;
@@ -118,6 +118,7 @@ static BwdPlan wide_plan(int64_t B, int64_t T, int64_t H, int64_t W, int tt_rows
 	if (group > 1 && !(p.branch_free && p.per <= (rank ? 4 : 8))) p.fast = false;  // grouped tiles: branch-free form only
 	p.deep = deep;
 	if (deep && !(p.branch_free && T % (2 * BWD_SJ) == 0)) p.fast = false;  // two-step prefetch: branch-free form only
+	if (deep == 2) p.lds_bytes *= 2;
 	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_groups * T * HW * sizeof(float) : 0;
 	p.rank_bytes = rank ? ((size_t)2 * T * HW + (size_t)(p.n_tt + 1) * T * H) * sizeof(float) : 0;
 	p.per_batch_bytes = p.partial_bytes + p.rank_bytes;
@@ -204,7 +205,7 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, const char* mode, int argc,
 		free(ws);
 		if (!rc && argc >= 8 && !strcmp(argv[4], "wide")) {
 			const BwdPlan p = wide_plan(B, T, H, W, atoi(argv[5]), atoi(argv[6]) != 0, atoi(argv[7]),
-			                            argc >= 9 && !strcmp(argv[8], "deep"));
+			                            argc < 9 ? 0 : !strcmp(argv[8], "deep") ? 1 : !strcmp(argv[8], "deep2") ? 2 : 0);
 			if (!p.fast) return 4;  // the kernels' limits rule this plan out
 			rc = run_wide(p, dA, q, k, dq, dk, B, T, H, W);
 		} else if (!rc) {

@@ -587,8 +587,9 @@ _Z4kernv: ; @k
 
 
 def test_backward_variants_are_chosen_by_the_environment_only(lib):
-    """L1ATTN_BWD_PREFETCH=2 turns the branch-free plans into their two-step-prefetch form and nothing else; it is
-    read once per process, hence the child process."""
+    """L1ATTN_BWD_PREFETCH=2 / =3 turn the branch-free plans into their pipelined forms (two steps of prefetch
+    distance; the same with two LDS planes, hence twice the LDS) and change nothing else; the variable is read
+    once per process, hence the child processes."""
     code = ("import ctypes, sys; L = ctypes.CDLL(sys.argv[1]);"
             "L.l1attn_dense_bwd_plan_info.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_void_p];"
             "out = [];\n"
@@ -597,11 +598,14 @@ def test_backward_variants_are_chosen_by_the_environment_only(lib):
             "print(out)")
     import _l1attn_hip as drv
     runs = {}
-    for depth in ("", "2"):
-        env = dict(os.environ, L1ATTN_BWD_PREFETCH=depth)
+    for value in ("", "2", "3", "7"):
+        env = dict(os.environ, L1ATTN_BWD_PREFETCH=value)
         r = subprocess.run([sys.executable, "-c", code, drv._LIB_PATH], env=env, capture_output=True, text=True, check=True)
-        runs[depth] = eval(r.stdout)
-    for one, two in zip(runs[""], runs["2"]):
-        assert one[14] == 0 and two[14] == one[3]            # exactly the branch-free plans change
-        assert one[:14] == two[:14]                          # and in nothing but that flag
-    assert [p[14] for p in runs["2"]] == [0, 1, 1, 0, 0]
+        runs[value] = eval(r.stdout)
+    assert runs["7"] == runs[""] and all(p[14] == 0 for p in runs[""])          # unknown values mean the default
+    for form, value in ((1, "2"), (2, "3")):
+        for one, two in zip(runs[""], runs[value]):
+            assert two[14] == form * one[3]                                      # exactly the branch-free plans change
+            assert two[11] == one[11] * (2 if two[14] == 2 else 1)               # LDS: two planes in form 2
+            assert one[:11] + one[12:14] == two[:11] + two[12:14]                # and nothing else
+    assert [p[14] for p in runs["3"]] == [0, 2, 2, 0, 0]

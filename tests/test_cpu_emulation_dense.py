@@ -143,16 +143,25 @@ def test_dense_backward_wide_tile_kernels(runner, tmp_path, shape, tt, rank, gro
     _check(_run(runner, tmp_path, shape, extra=("wide", tt, rank, group), seed=sum(shape) + tt, ties=ties), 1e-5, 1e-4)
 
 
-@pytest.mark.parametrize("shape,rank,group", [((2, 128, 2, 64), 0, 1), ((2, 128, 2, 64), 1, 1), ((3, 128, 4, 64), 0, 2),
-                                              ((1, 256, 4, 64), 1, 4), ((1, 64, 1, 64), 1, 1)])
-def test_two_step_prefetch_equals_the_one_step_loop(runner, tmp_path, shape, rank, group):
-    """dense_bwd_f32_fast<..., DEEP>: two register sets of prefetched values alternate and the step loop runs two
-    steps per iteration.  Same sums in the same order: dq and dk equal the one-step loop's bit for bit (and the
-    oracle's within the usual tolerance), also where the sequence is a single pair of steps short of nothing
-    (64 tokens = sixteen steps) and with half-integer inputs (ties)."""
-    deep = _run(runner, tmp_path, shape, extra=("wide", 64, rank, group, "deep"), seed=5, ties=bool(rank))
+_ONE_STEP = {}  # results of the one-step loop, shared by the two forms compared with it
+
+
+@pytest.mark.parametrize("form", ["deep", "deep2"])
+@pytest.mark.parametrize("shape,rank,group", [((2, 128, 2, 64), 0, 1), ((1, 128, 2, 64), 1, 1), ((3, 128, 2, 64), 0, 2),
+                                              ((1, 256, 2, 64), 1, 4), ((1, 64, 1, 64), 1, 1)])
+def test_pipelined_step_loops_equal_the_one_step_loop(runner, tmp_path, shape, rank, group, form):
+    """dense_bwd_f32_fast<..., DEEP>.  "deep": two register sets of prefetched values alternate and the step loop
+    runs two steps per iteration.  "deep2": the two steps also stage their tiles in two LDS planes and keep one
+    barrier each.  Same sums in the same order: dq and dk equal the one-step loop's bit for bit (and the oracle's
+    within the usual tolerance), also at the shortest sequence (64 tokens = sixteen steps), over several tiles per
+    workgroup (where the rank form's row sums of one tile are read from the plane the next tile writes first) and
+    with half-integer inputs (ties)."""
+    deep = _run(runner, tmp_path, shape, extra=("wide", 64, rank, group, form), seed=5, ties=bool(rank))
     _check(deep, 1e-5, 1e-4)
-    one = _run(runner, tmp_path, shape, extra=("wide", 64, rank, group), seed=5, ties=bool(rank))
+    key = (shape, rank, group)
+    if key not in _ONE_STEP:
+        _ONE_STEP[key] = _run(runner, tmp_path, shape, extra=("wide", 64, rank, group), seed=5, ties=bool(rank))
+    one = _ONE_STEP[key]
     assert torch.equal(deep["dq"], one["dq"]) and torch.equal(deep["dk"], one["dk"])
 
 
@@ -184,6 +193,10 @@ def test_dense_kernels_under_thread_sanitizer(tmp_path, emu_dense_tsan):
     _check(_run(exe, d, (1, 136, 2, 64), extra=("wide", 72, 0, 1), seed=4), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 128, 4, 64), extra=("wide", 64, 1, 2, "deep"), seed=6), 1e-5, 1e-4)
     _check(_run(exe, d, (2, 64, 2, 64), extra=("wide", 64, 0, 1, "deep"), seed=7), 1e-5, 1e-4)
+    # one barrier per step, two LDS planes: the rank form over several tiles per workgroup is the case that needs
+    # the extra barrier per tile (found here: without it the next tile's first write races the row-sum reads)
+    _check(_run(exe, d, (1, 256, 2, 64), extra=("wide", 64, 1, 4, "deep2"), seed=8), 1e-5, 1e-4)
+    _check(_run(exe, d, (3, 128, 2, 64), extra=("wide", 64, 0, 2, "deep2"), seed=9), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 64, 2, 64), mode="fixed", seed=5), 1e-5, None)
 
 

@@ -44,10 +44,10 @@ def _today(name):
     m = re.match(r"(sparse\.hip sparse_\w+)<(float|double), (.*)>$", name)
     if m:
         return "%s<%s, %s, %s>" % (m.group(1), m.group(2), m.group(3), m.group(2))
-    # the tiled dense backward gained a last template flag (two steps of prefetch distance); the tested kernels
-    # are the instantiations with the flag off
+    # the tiled dense backward gained a last template argument (the form of the branch-free step loop); the tested
+    # kernels are the instantiations of form 0
     m = re.match(r"(dense\.hip dense_bwd_f32_fast)<(.*)>$", name)
-    return "%s<%s, false>" % (m.group(1), m.group(2)) if m else name
+    return "%s<%s, 0>" % (m.group(1), m.group(2)) if m else name
 
 
 def test_gpu_tested_kernels_are_unchanged():

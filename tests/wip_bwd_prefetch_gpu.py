@@ -1,6 +1,7 @@
-"""GPU parity of the dense backward's two-step-prefetch step loop (csrc/dense.hip, dense_bwd_f32_fast<..., DEEP>)
-against the one-step form the backward uses by default: the same sums in the same order, so dq and dk must be
-equal bit for bit, in all four branch-free instantiations (sign or rank form, one or several tiles per workgroup).
+"""GPU parity of the dense backward's pipelined step loops (csrc/dense.hip, dense_bwd_f32_fast<..., DEEP>: two steps
+of prefetch distance, and the same with two LDS planes and one barrier per step) against the one-step form the
+backward uses by default: the same sums in the same order, so dq and dk must be equal bit for bit, in the sign and
+the rank form, with one or several tiles per workgroup.
 
 This file has not run on a GPU yet, which is why its name keeps it out of pytest's collection
 (run it as `python -m pytest tests/wip_bwd_prefetch_gpu.py -m gpu`); rename it to test_*.py once it has passed there.
@@ -38,12 +39,14 @@ def test_two_step_prefetch_equals_the_default_backward(tmp_path, shape, kind):
         "torch.save([dq.cpu(), dk.cpu(), torch.tensor(list(info))], sys.argv[1])"
         % (os.path.join(ROOT, "l1-attention_amd"), shape))
     outs = []
-    for name, env in (("one_step", {}), ("two_steps", {"L1ATTN_BWD_PREFETCH": "2"})):
+    for name, env in (("one_step", {}), ("two_steps", {"L1ATTN_BWD_PREFETCH": "2"}),
+                      ("two_steps_two_planes", {"L1ATTN_BWD_PREFETCH": "3"})):
         path = str(tmp_path / (name + ".pt"))
         print("case backward with prefetch distance:", name, shape, flush=True)
         subprocess.run([sys.executable, "-c", code, path], check=True, env=dict(os.environ, **env), timeout=300)
         outs.append(torch.load(path, weights_only=True))
-    (dq1, dk1, plan1), (dq2, dk2, plan2) = outs
-    assert int(plan1[3]) == 1 and int(plan1[14]) == 0 and int(plan2[14]) == 1          # branch-free; one step / two steps
+    (dq1, dk1, plan1), (dq2, dk2, plan2), (dq3, dk3, plan3) = outs
+    assert int(plan1[3]) == 1 and [int(p[14]) for p in (plan1, plan2, plan3)] == [0, 1, 2]   # branch-free; the three forms
     assert (int(plan2[2]), int(int(plan2[9]) > 1)) == kind
     assert torch.equal(dq1, dq2) and torch.equal(dk1, dk2)
+    assert torch.equal(dq1, dq3) and torch.equal(dk1, dk3)
