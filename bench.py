@@ -113,6 +113,15 @@ def dense_headline(steps, warmup):
         "fwd_bwd_gops": 6 * N / (ms_per_step * 1e-3) / 1e9,
     }
     out["frac_of_valu_peak"] = out["fwd_bwd_gops"] / 1e3 / P_VALU_TOPS
+    # which forms of the backward this process ran (both are chosen from the environment, read once by the library)
+    import ctypes
+    import _l1attn_hip as drv
+    info = (ctypes.c_int64 * 16)()
+    drv.lib().l1attn_dense_bwd_plan_info(B, T, H, W, info)
+    out["backward_plan"] = {"rank_form": int(info[2]), "branch_free": int(info[3]), "tiles_per_workgroup": int(info[9]),
+                            "step_loop_form": int(info[14]),
+                            "L1ATTN_BWD_PREFETCH": os.environ.get("L1ATTN_BWD_PREFETCH"),
+                            "L1ATTN_RANK_SORT": os.environ.get("L1ATTN_RANK_SORT")}
     del dA, q, k
     torch.cuda.empty_cache()
     return out
