@@ -165,6 +165,35 @@ def test_pipelined_step_loops_equal_the_one_step_loop(runner, tmp_path, shape, r
     assert torch.equal(deep["dq"], one["dq"]) and torch.equal(deep["dk"], one["dk"])
 
 
+def test_all_tie_column_in_the_rank_form(runner, tmp_path):
+    """A column in which every q equals every k has sign(q - k) = 0 throughout: the reference's gradients there are
+    exactly zero (cpp/l1attn_drv.cpp:7-11).  The sign form reproduces the zeros; the rank form computes
+    2 * sum(hv * g) - sum(g) with hv = 1/2, which leaves the rounding residue of the two sums.  This pins the size
+    of that residue: below 1e-5 of the largest gradient, the forward tolerance."""
+    B, T, H, W = 1, 128, 2, 64
+    g = torch.Generator().manual_seed(31)
+    q, k = torch.randn(B, T, H, W, generator=g), torch.randn(B, T, H, W, generator=g)
+    q[..., 5] = k[..., 5] = 0.75
+    dA = torch.randn(B, T, T, H, generator=g)
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    res = {}
+    for rank in (0, 1):
+        with open(fin, "wb") as f:
+            f.write(struct.pack("4q", B, T, H, W))
+            for x in (q, k, dA):
+                f.write(x.numpy().tobytes())
+        r = subprocess.run([runner, fin, fout, "f32", "wide", "64", str(rank), "1"], env=ENV, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        raw = np.fromfile(fout, np.float32, count=B * T * T * H + 2 * B * T * H * W)[B * T * T * H:]
+        res[rank] = torch.from_numpy(raw.copy()).view(2, B, T, H, W)
+    rdq, rdk = oracle.dense_bwd(dA.double(), q.double(), k.double())
+    assert float(rdq[..., 5].abs().max()) == 0.0 and float(rdk[..., 5].abs().max()) == 0.0
+    assert float(res[0][..., 5].abs().max()) == 0.0                                  # sign form: exact zeros
+    big = float(max(rdq.abs().max(), rdk.abs().max()))
+    assert 0.0 < float(res[1][..., 5].abs().max()) <= 1e-5 * big                      # rank form: a residue, this small
+    assert cf.rel_err(res[1][0], rdq) <= 1e-4 and cf.rel_err(res[1][1], rdk) <= 1e-4
+
+
 def test_plans_outside_the_kernels_limits_are_refused(runner, tmp_path):
     """The runner's plan builder mirrors the library's limits: sixteen lanes per staged (src row, head) in the rank
     form, at most eight staged values per thread."""
