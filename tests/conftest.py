@@ -32,7 +32,7 @@ CLANG = "/opt/rocm/llvm/bin/clang++"
 RUNNERS = {"fused": ("fused", "g++", "address,undefined"), "sparse": ("sparse", CLANG, "address,undefined"),
            "ranks": ("ranks", "g++", "address,undefined"), "dense": ("dense", "g++", "address,undefined"),
            "fused_tsan": ("fused", "g++", "thread"), "sparse_tsan": ("sparse", CLANG, "thread"),
-           "dense_tsan": ("dense", "g++", "thread")}
+           "dense_tsan": ("dense", "g++", "thread"), "ranks_tsan": ("ranks", "g++", "thread")}
 
 
 @pytest.fixture(scope="session")
@@ -96,3 +96,8 @@ def emu_sparse_tsan(_emu_builds):
 @pytest.fixture(scope="session")
 def emu_dense_tsan(_emu_builds):
     return _emu_runner(_emu_builds, "dense_tsan")
+
+
+@pytest.fixture(scope="session")
+def emu_ranks_tsan(_emu_builds):
+    return _emu_runner(_emu_builds, "ranks_tsan")

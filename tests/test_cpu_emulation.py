@@ -287,3 +287,25 @@ def test_merge_sort_column_ranks_on_cpu(tmp_path, shape, ranks_runner):
         hv = np.clip(rq[:, :, None] - rk[:, None], 0.0, 1.0)             # [B,T(dst),S(src),H,W]
         sign = np.sign((q.numpy()[:, :, None] + 0.0) - (k.numpy()[:, None] + 0.0))
         assert np.array_equal(2 * hv - 1, sign)
+
+
+@pytest.mark.parametrize("shape", [(1, 1000, 1, 2), (1, 2049, 1, 1)])
+def test_merge_sort_column_ranks_have_no_data_race(tmp_path, shape, emu_ranks_tsan):
+    """The merge rounds work in place in LDS: every thread reads its inputs, a barrier, every thread writes its
+    outputs, a barrier.  Under ThreadSanitizer a thread that wrote before another had read would be a data race."""
+    B, T, H, W = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    with open(fin, "wb") as f:
+        f.write(struct.pack("4q", B, T, H, W))
+        f.write(q.numpy().tobytes())
+        f.write(k.numpy().tobytes())
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 report_signal_unsafe=0")
+    r = subprocess.run([emu_ranks_tsan, fin, fout], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, (r.returncode, r.stderr[:3000])
+    n = B * T * H * W
+    raw = open(fout, "rb").read()
+    ref_rq, ref_rk = _reference_ranks(q, k)
+    assert np.array_equal(np.frombuffer(raw, np.float32, n).reshape(B, T, H, W), ref_rq)
+    assert np.array_equal(np.frombuffer(raw, np.float32, n, n * 4).reshape(B, T, H, W), ref_rk)
