@@ -218,7 +218,9 @@ def check_hot_kernels(res):
     want = {  # substring of the mangled name -> most VGPRs per lane
         "dense_fwd_f32_pipeILi64E": 128,                              # 1024 threads: four waves per SIMD
         "dense_fwd_f32_pipeILi32E": 128,
-        "dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E": 256,        # 512 threads: two waves per SIMD
+        "dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E": 256,        # 512 threads: two waves per SIMD (all loop forms)
+        "dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb0ELb1E": 256,
+        "dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb1ELb1E": 256,
         "dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1E": 256,
         "dense_bwd_reduce_dkILb1ELb1E": 64,
     }
@@ -278,8 +280,13 @@ def loop_profiles(asm_text, kernel_substr):
 HOT_LOOPS = (
     ("dense_fwd_f32_pipeILi64ELb0E", 8 * 64, 2, 2.30),                    # eight src rows of 64 columns per lane
     ("dense_fwd_f32_pipeILi32ELb0E", 8 * 32, 2, 2.55),
-    ("dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E", 4 * 64, 3, 3.20),  # four src rows against 64 dst tokens, ranks
-    ("dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1E", 4 * 64, 4, 4.25),  # the same with the sign from the difference
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1ELi0E", 4 * 64, 3, 3.20),  # four src rows against 64 dst tokens, ranks
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1ELi0E", 4 * 64, 4, 4.25),  # the same with the sign from the difference
+    # the pipelined forms of the same loops: two steps per iteration
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1ELi1E", 8 * 64, 3, 3.20),
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1ELi2E", 8 * 64, 3, 3.20),
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1ELi1E", 8 * 64, 4, 4.25),
+    ("dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1ELi2E", 8 * 64, 4, 4.25),
 )
 
 

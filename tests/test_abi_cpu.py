@@ -323,6 +323,8 @@ amdhsa.target:   amdgcn-amd-amdhsa--gfx950
             "k_dense_fwd_f32_pipeILi32E": dict(vgpr=70, scratch_bytes=0, vgpr_spills=0),
             "k_dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb1ELb1E": dict(vgpr=218, scratch_bytes=0, vgpr_spills=0),
             "k_dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb0ELb1E": dict(vgpr=190, scratch_bytes=0, vgpr_spills=0),
+            "k_dense_bwd_f32_fastILi64ELi512ELi4ELb1ELb0ELb1E": dict(vgpr=220, scratch_bytes=0, vgpr_spills=0),
+            "k_dense_bwd_f32_fastILi64ELi512ELi4ELb0ELb1ELb1E": dict(vgpr=187, scratch_bytes=0, vgpr_spills=0),
             "k_dense_bwd_reduce_dkILb1ELb1E": dict(vgpr=20, scratch_bytes=0, vgpr_spills=0)}
     build.check_hot_kernels(full)
     for name, change in [("k_dense_fwd_f32_pipeILi64E", dict(vgpr=130)),              # three waves per SIMD only
