@@ -160,14 +160,18 @@ static int run_wide(const BwdPlan& p, const float* d_attn, const float* q, const
 		}
 		const bool vec = ((T * HW) % 4 == 0) && ((((uintptr_t)dkp) | ((uintptr_t)dk)) & 15) == 0 && (!p.rank || W % 4 == 0);
 		const dim3 rgrid((unsigned)l1_cdiv(ne, vec ? 1024 : 256));
-#define RUN_REDUCE(VECV, RANKV)                                                                                       \
-	hipLaunchKernelGGL((dense_bwd_reduce_dk<VECV, RANKV>), rgrid, dim3(256), 0, st, dkp, dk + b0 * T * HW, ne, p.n_groups, \
-	                   cs, (int)HW, (int)W, (int)H, scale)
-		if (vec && p.rank) RUN_REDUCE(true, true);
+#define RUN_REDUCE3(VECV, RANKV, AHEADV)                                                                              \
+	hipLaunchKernelGGL((dense_bwd_reduce_dk<VECV, RANKV, AHEADV>), rgrid, dim3(256), 0, st, dkp, dk + b0 * T * HW, ne,     \
+	                   p.n_groups, cs, (int)HW, (int)W, (int)H, scale)
+#define RUN_REDUCE(VECV, RANKV) RUN_REDUCE3(VECV, RANKV, false)
+		if (vec && p.deep && p.rank) RUN_REDUCE3(true, true, true);
+		else if (vec && p.deep) RUN_REDUCE3(true, false, true);
+		else if (vec && p.rank) RUN_REDUCE(true, true);
 		else if (vec) RUN_REDUCE(true, false);
 		else if (p.rank) RUN_REDUCE(false, true);
 		else RUN_REDUCE(false, false);
 #undef RUN_REDUCE
+#undef RUN_REDUCE3
 	}
 	free(workspace);
 	return 0;

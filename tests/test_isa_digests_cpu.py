@@ -47,7 +47,11 @@ def _today(name):
     # the tiled dense backward gained a last template argument (the form of the branch-free step loop); the tested
     # kernels are the instantiations of form 0
     m = re.match(r"(dense\.hip dense_bwd_f32_fast)<(.*)>$", name)
-    return "%s<%s, 0>" % (m.group(1), m.group(2)) if m else name
+    if m:
+        return "%s<%s, 0>" % (m.group(1), m.group(2))
+    # and its reduction kernel a flag for reading several partial arrays ahead, off in the tested kernels
+    m = re.match(r"(dense\.hip dense_bwd_reduce_dk)<(.*)>$", name)
+    return "%s<%s, false>" % (m.group(1), m.group(2)) if m else name
 
 
 def test_gpu_tested_kernels_are_unchanged():
