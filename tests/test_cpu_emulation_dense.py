@@ -30,8 +30,8 @@ ENV = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0",
            TSAN_OPTIONS="halt_on_error=1 report_signal_unsafe=0")
 
 
-def _run(exe, d, shape, mode="f32", extra=(), seed=0, ties=False, scale=1.0):
-    """-> dict with attn, dq, dk (as far as the mode has them), plan, and the inputs."""
+def _run(exe, d, shape, mode="f32", extra=(), seed=0, ties=False, scale=1.0, inputs=None):
+    """-> dict with attn, dq, dk (as far as the mode has them), plan, and the inputs (seeded, or `inputs` = q, k, dA)."""
     B, T, H, W = shape
     dt = torch.float64 if mode == "f64" else torch.float32
     g = torch.Generator().manual_seed(seed)
@@ -39,6 +39,8 @@ def _run(exe, d, shape, mode="f32", extra=(), seed=0, ties=False, scale=1.0):
     if ties:  # half-integers: exact ties between q and k, and among the k of a column
         q, k = torch.round(q * 2) / 2, torch.round(k * 2) / 2
     dA = torch.randn(B, T, T, H, generator=g, dtype=dt)
+    if inputs is not None:
+        q, k, dA = (x.to(dt).contiguous() for x in inputs)
     fin, fout = str(d / "in.bin"), str(d / "out.bin")
     with open(fin, "wb") as f:
         f.write(struct.pack("4q", B, T, H, W))
@@ -117,6 +119,26 @@ def test_dense_float64_and_ties(runner, tmp_path):
     assert float((r["q"][:, :, None] == r["k"][:, None]).float().mean()) > 0.1  # sign(0) = 0 matters here
     _check(r, 1e-6, 1e-5)
     _check(_run(runner, tmp_path, (1, 33, 2, 7), ties=True, seed=9), 1e-6, 1e-5)  # untiled kernels, exact compares
+
+
+def test_dense_kernels_against_the_reference_extension_golden_vectors(runner, tmp_path):
+    """tests/golden/ref_cpp_golden.npz holds inputs and outputs of the reference's own compiled CPU extension
+    (cpp/l1attn_drv.cpp; written by tests/golden/make_golden.py), with exact ties planted.  The float64 kernels sum
+    in the reference's order: equal to the last bit.  The float32 kernels on the same inputs: the usual tolerances."""
+    z = np.load(os.path.join(HERE, "golden", "ref_cpp_golden.npz"))
+    for tag in ("dA", "dB"):
+        q, k, da = (torch.from_numpy(z["%s_%s" % (tag, n)]) for n in ("q", "k", "da"))
+        want = [torch.from_numpy(z["%s_%s" % (tag, n)]) for n in ("attn", "dq", "dk")]
+        r = _run(runner, tmp_path, tuple(q.shape), mode="f64", inputs=(q, k, da))
+        for name, w in zip(("attn", "dq", "dk"), want):
+            assert torch.equal(r[name], w), (tag, name)
+        r = _run(runner, tmp_path, tuple(q.shape), mode="f32", inputs=(q, k, da))
+        f32_in = [x.float().double() for x in (q, k)]  # what the float32 kernels were given
+        assert cf.rel_err(r["attn"], oracle.dense_fwd(*f32_in)) <= 1e-5
+        assert cf.rel_err(r["attn"], want[0]) <= 1e-5 and cf.rel_err(r["dk"], want[2]) <= 1e-4
+        # (dq, dk of float32-rounded inputs may differ from the float64 golden where a tie is broken by the rounding)
+        rdq, rdk = oracle.dense_bwd(da.float().double(), *f32_in)
+        assert cf.rel_err(r["dq"], rdq) <= 1e-4 and cf.rel_err(r["dk"], rdk) <= 1e-4
 
 
 WIDE_CASES = [

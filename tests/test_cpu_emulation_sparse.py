@@ -186,3 +186,19 @@ def test_sparse_kernels_under_thread_sanitizer(tmp_path, emu_sparse_tsan):
         x = [t.double() for t in (vf, vb, q, k)]
         ref = cf.bidi_value(*x, co, True) if bidi else cf.sparse_value(x[0], x[2], x[3], co, True)
         assert cf.rel_err(vo, ref) <= (1e-5 if kind == "f32" else TOL[kind])
+
+
+def test_sparse_kernels_against_the_reference_extension_golden_vectors(runner, tmp_path):
+    """Forward outputs of the reference's own compiled CPU extension (tests/golden/ref_cpp_golden.npz, written by
+    tests/golden/make_golden.py: both edge lists, both `use_softmax`, one-directional and bidirectional) against
+    the float64 kernels.  The runner takes its inputs as float32, so the comparison is at the rounding of the inputs
+    (1e-6 of the largest output), not at the last bit."""
+    z = np.load(os.path.join(HERE, "golden", "ref_cpp_golden.npz"))
+    for tag in ("sA", "sB"):
+        co = torch.from_numpy(z[tag + "_co"])
+        v, vb, q, k = (torch.from_numpy(z["%s_%s" % (tag, n)]).float() for n in ("v", "vb", "q", "k"))
+        for sm, name in ((True, "sm"), (False, "nsm")):
+            vo, _, _ = _run(runner, tmp_path, v, vb, q, k, co, sm, False, "f64")
+            assert cf.rel_err(vo, torch.from_numpy(z["%s_%s_vo" % (tag, name)])) <= 1e-6, (tag, name)
+            vo, _, _ = _run(runner, tmp_path, v, vb, q, k, co, sm, True, "f64")
+            assert cf.rel_err(vo, torch.from_numpy(z["%s_%s_bidi_vo" % (tag, name)])) <= 1e-6, (tag, name, "bidi")
