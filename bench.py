@@ -256,6 +256,11 @@ def extra_legs():
         def fused_step():
             train(lambda: fused(*x))
 
+        fused_piped = l1attn_cuda.L1AttnFused(pipelined=True)
+
+        def fused_piped_step():
+            train(lambda: fused_piped(*x))
+
         def composed_step():
             def f():
                 a = plain(x[0], x[1])
@@ -264,7 +269,7 @@ def extra_legs():
             train(f)
 
         steps = {}
-        for label, fn in (("fused", fused_step), ("composed", composed_step)):
+        for label, fn in (("fused", fused_step), ("fused_pipelined", fused_piped_step), ("composed", composed_step)):
             torch.cuda.empty_cache()
             torch.cuda.reset_peak_memory_stats()
             base = torch.cuda.memory_allocated()

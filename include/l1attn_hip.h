@@ -184,6 +184,14 @@ int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k,
 int l1attn_fused_bwd_stage_f64(const double* dvo, const double* q, const double* k, const double* v,
                                const double* vo, const double* lse, double* dA, double* dv,
                                int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
+/*
+ * l1attn_fused_bwd_stage_f32 with the wave-uniform rows of both kernels streamed through a software pipeline of
+ * scalar loads where such kernels exist (W == Wv in {32, 64}; other shapes run what l1attn_fused_bwd_stage_f32
+ * runs).  Same arithmetic in the same order: bit-equal dA and dv.  No counterpart in the reference.
+ */
+int l1attn_fused_bwd_stage_pipe_f32(const float* dvo, const float* q, const float* k, const float* v,
+                                    const float* vo, const float* lse, float* dA, float* dv,
+                                    int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv, void* stream);
 
 /* -------------------------------------------------------------------------- edge lists */
 

@@ -95,6 +95,9 @@ def lib():
             f = getattr(L, "l1attn_fused_bwd_stage_" + sfx)
             f.restype = _c_i
             f.argtypes = [_c_p] * 8 + [_c_i64] * 5 + [_c_p]
+            if sfx == "f32":
+                L.l1attn_fused_bwd_stage_pipe_f32.restype = _c_i
+                L.l1attn_fused_bwd_stage_pipe_f32.argtypes = f.argtypes
         L.l1attn_dense_column_ranks_f32.restype = _c_i
         L.l1attn_dense_column_ranks_f32.argtypes = [_c_p] * 4 + [_c_i64] * 4 + [_c_p]
         L.l1attn_dense_column_ranks_merge_f32.restype = _c_i
@@ -290,8 +293,9 @@ def fused_backward_slab(B, T, H, itemsize):
     return max(1, min(B, _fused_da_bytes // per_entry if per_entry else B))
 
 
-def dense_fused_backward(dvo, q, k, v, vo, lse):
-    """Backward of dense_fused_forward -> [dq, dk, dv].  Stage one writes dA (the gradient of the logits, from
+def dense_fused_backward(dvo, q, k, v, vo, lse, pipelined=False):
+    """Backward of dense_fused_forward -> [dq, dk, dv].  pipelined: the first stage through
+    l1attn_fused_bwd_stage_pipe_f32 (float32 only; same results bit for bit).  Stage one writes dA (the gradient of the logits, from
     dvo and the forward's vo and lse) and dv; dq and dk are the dense backward of dA.  Batch entries are
     independent, so the batch goes through in slabs that share one dA buffer of [slab,T,T,H] (stream order
     keeps a slab's readers ahead of the next slab's writer): the whole [B,T,T,H] tensor never exists, 1 GiB in place
@@ -310,25 +314,26 @@ def dense_fused_backward(dvo, q, k, v, vo, lse):
         raise RuntimeError("v must have the dtype and device of q, and lse must be the [batch, n_ctx, n_heads] "
                            "tensor the forward returned")
     sfx = sfx_of(q)
+    stage = "l1attn_fused_bwd_stage_pipe_f32" if (pipelined and sfx == "f32") else "l1attn_fused_bwd_stage_" + sfx
     slab = fused_backward_slab(B, T, H, q.element_size())
     dA = torch.empty((slab, T, T, H), dtype=q.dtype, device=q.device)
     dv = torch.empty_like(v)
     if slab >= B:
         with torch.cuda.device(q.device):
-            rc = getattr(lib(), "l1attn_fused_bwd_stage_" + sfx)(
+            rc = getattr(lib(), stage)(
                 ptr(dvo), ptr(q), ptr(k), ptr(v), ptr(vo), ptr(lse), ptr(dA), ptr(dv), B, T, H, W, v.shape[3],
                 stream_of(q))
-        check(rc, "l1attn_fused_bwd_stage_" + sfx)
+        check(rc, stage)
         dq, dk = dense_backward(dA, q, k)
         return [dq, dk, dv]
     dq, dk = torch.empty_like(q), torch.empty_like(k)
     for b0 in range(0, B, slab):
         b1 = min(B, b0 + slab)  # (a slice of leading batch entries of a contiguous tensor is contiguous)
         with torch.cuda.device(q.device):
-            rc = getattr(lib(), "l1attn_fused_bwd_stage_" + sfx)(
+            rc = getattr(lib(), stage)(
                 ptr(dvo[b0:b1]), ptr(q[b0:b1]), ptr(k[b0:b1]), ptr(v[b0:b1]), ptr(vo[b0:b1]), ptr(lse[b0:b1]), ptr(dA),
                 ptr(dv[b0:b1]), b1 - b0, T, H, W, v.shape[3], stream_of(q))
-        check(rc, "l1attn_fused_bwd_stage_" + sfx)
+        check(rc, stage)
         dq[b0:b1], dk[b0:b1] = dense_backward(dA[:b1 - b0], q[b0:b1], k[b0:b1])
     return [dq, dk, dv]
 

@@ -125,10 +125,19 @@ __global__ __launch_bounds__(256) void fused_fwd_f32_tile(const float* __restric
 // of the next row, clamped to the last row at the end (read, never used), and drained after the loop.
 
 // Chunk C of a src token's 2*W/32 (k chunks first, then v chunks), then the chunks after it.
-template <int W, int C>
-__device__ __forceinline__ void fused_pipe_chunks(const float (&qr)[W], float (&acc)[W], float& a, float& p, float& den,
+// The three sweeps of the fused operator share this stream; what differs is what the second row's chunks do:
+//   FUSED_FWD  xr = q row, rows = k, v:    a += |xr - k|;  p = e^{a*scale}, den += p;  yr (vo sums) += p * v
+//   FUSED_DV   xr = k row, rows = q, dvo:  a += |xr - q|;  p = e^{a*scale - l};         yr (dv sums) += p * dvo
+//   FUSED_DA   xr = q row, rows = k, v:    a += |xr - k|;  p (a dot product) += yr (dvo row) * v
+// l (FUSED_DV): the dst token's lse, a scalar the compiler loads; `pin` names the next token's, whose load the
+// caller has just issued: it is taken right after this chunk's wait, where nothing is in flight, so that the
+// compiler's own wait for it never falls between a prefetch and the work that covers it.
+enum { FUSED_FWD = 0, FUSED_DV = 1, FUSED_DA = 2 };
+template <int W, int C, int ROLE = FUSED_FWD>
+__device__ __forceinline__ void fused_pipe_chunks(const float (&xr)[W], float (&yr)[W], float& a, float& p, float& den,
                                                   float scale, f32x16& b0l, f32x16& b0h, f32x16& b1l, f32x16& b1h,
-                                                  const float* krow, const float* vrow, const float* knext)
+                                                  const float* krow, const float* vrow, const float* knext,
+                                                  float l = 0.0f, float* pin = nullptr)
 {
 	constexpr int CPR = W / 32;  // chunks per k row and per v row
 	f32x16& lo = (C & 1) == 0 ? b0l : b1l;  // this chunk's buffer
@@ -139,6 +148,7 @@ __device__ __forceinline__ void fused_pipe_chunks(const float (&qr)[W], float (&
 	// come a few instructions after the load it waits for)
 	__builtin_amdgcn_sched_barrier(0);
 	swait32(lo, hi);
+	if constexpr (ROLE == FUSED_DV && C == 0) sarrived(*pin);
 	__builtin_amdgcn_sched_barrier(0);
 	// the chunk after this one: the rest of the k row, then the v row, then the next token's k row
 	if constexpr (C + 1 < CPR) sload32_at<(C + 1) * 128>(nl, nh, krow);
@@ -147,21 +157,30 @@ __device__ __forceinline__ void fused_pipe_chunks(const float (&qr)[W], float (&
 	__builtin_amdgcn_sched_barrier(0);
 	if constexpr (C < CPR) {
 #pragma unroll
-		for (int i = 0; i < 16; i++) a += fabsf(qr[C * 32 + i] - lo[i]);
+		for (int i = 0; i < 16; i++) a += fabsf(xr[C * 32 + i] - lo[i]);
 #pragma unroll
-		for (int i = 0; i < 16; i++) a += fabsf(qr[C * 32 + 16 + i] - hi[i]);
+		for (int i = 0; i < 16; i++) a += fabsf(xr[C * 32 + 16 + i] - hi[i]);
+	} else if constexpr (ROLE == FUSED_DA) {
+#pragma unroll
+		for (int i = 0; i < 16; i++) p += yr[(C - CPR) * 32 + i] * lo[i];
+#pragma unroll
+		for (int i = 0; i < 16; i++) p += yr[(C - CPR) * 32 + 16 + i] * hi[i];
 	} else {
 		if constexpr (C == CPR) {
-			p = expf(a * scale);
-			den += p;
+			if constexpr (ROLE == FUSED_FWD) {
+				p = expf(a * scale);
+				den += p;
+			} else {
+				p = expf(a * scale - l);
+			}
 		}
 #pragma unroll
-		for (int i = 0; i < 16; i++) acc[(C - CPR) * 32 + i] += p * lo[i];
+		for (int i = 0; i < 16; i++) yr[(C - CPR) * 32 + i] += p * lo[i];
 #pragma unroll
-		for (int i = 0; i < 16; i++) acc[(C - CPR) * 32 + 16 + i] += p * hi[i];
+		for (int i = 0; i < 16; i++) yr[(C - CPR) * 32 + 16 + i] += p * hi[i];
 	}
 	if constexpr (C + 1 < 2 * CPR)
-		fused_pipe_chunks<W, C + 1>(qr, acc, a, p, den, scale, b0l, b0h, b1l, b1h, krow, vrow, knext);
+		fused_pipe_chunks<W, C + 1, ROLE>(xr, yr, a, p, den, scale, b0l, b0h, b1l, b1h, krow, vrow, knext, l, pin);
 }
 
 template <int W>
@@ -400,6 +419,139 @@ __global__ __launch_bounds__(256) void fused_bwd_dv_tile(const float* __restrict
 	}
 }
 
+// Software-pipelined variants of the two tiled kernels above for W a multiple of 32 (see fused_fwd_f32_pipe): the
+// same mapping and the same arithmetic in the same order, the wave-uniform rows streamed through the two SGPR
+// buffers of sload.h instead of being loaded where the compiler puts them.
+
+template <int W>
+__global__ __launch_bounds__(64 * DA_NH) void fused_bwd_da_pipe(const float* __restrict__ dvo,
+                                                                  const float* __restrict__ q,
+                                                                  const float* __restrict__ k,
+                                                                  const float* __restrict__ v,
+                                                                  const float* __restrict__ vo,
+                                                                  const float* __restrict__ lse,
+                                                                  float* __restrict__ dA, int Tn, int H, int n_hg,
+                                                                  int NH, float scale)
+{
+	static_assert(W % 32 == 0, "whole 32-float chunks");
+	__shared__ float tile[DA_SJ][64 * (DA_NH + 1)];
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.y / n_hg, hg = lb.y % n_hg;
+	const int h = min(hg * NH + wave, H - 1);
+	const int t0 = lb.x * 64;
+	const int t = min(t0 + lane, Tn - 1);
+	const int PH = NH + 1;
+
+	float qr[W], gr[W];
+	float S = 0.0f;
+	{
+		const int64_t off = (((int64_t)b * Tn + t) * H + h) * (int64_t)W;
+		const float4* qp = reinterpret_cast<const float4*>(q + off);
+		const float4* gp = reinterpret_cast<const float4*>(dvo + off);
+		const float4* op = reinterpret_cast<const float4*>(vo + off);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = qp[w4], g = gp[w4], o = op[w4];
+			qr[w4 * 4 + 0] = x.x; qr[w4 * 4 + 1] = x.y; qr[w4 * 4 + 2] = x.z; qr[w4 * 4 + 3] = x.w;
+			gr[w4 * 4 + 0] = g.x; gr[w4 * 4 + 1] = g.y; gr[w4 * 4 + 2] = g.z; gr[w4 * 4 + 3] = g.w;
+			S += o.x * g.x; S += o.y * g.y; S += o.z * g.z; S += o.w * g.w;
+		}
+	}
+	float l = lse[((int64_t)b * Tn + t) * H + h];
+	// take the rows, S and lse here, before the first scalar prefetch is in flight
+#pragma unroll
+	for (int w = 0; w < W; w++) asm volatile("" : "+v"(qr[w]), "+v"(gr[w]));
+	asm volatile("" : "+v"(S), "+v"(l));
+	const int64_t row = (int64_t)H * W;
+	const float* const kb = k + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	const float* const vb = v + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	const int o_t = threadIdx.x / NH, o_h = threadIdx.x % NH;
+	const bool o_ok = (t0 + o_t < Tn) && (hg * NH + o_h < H);
+	float* const o_base = dA + (((int64_t)b * Tn) * Tn + (t0 + o_t)) * H + hg * NH + o_h;
+	const int64_t pitch = (int64_t)Tn * H;
+	float unused = 0.0f;
+	f32x16 b0l, b0h, b1l, b1h;
+	sload32(b0l, b0h, kb);
+	__builtin_amdgcn_sched_barrier(0);
+	for (int s0 = 0; s0 < Tn; s0 += DA_SJ) {
+#pragma unroll 1
+		for (int j = 0; j < DA_SJ; j++) {
+			// rows past the end are computed on the last row and not stored; the row after it is the next in the stream
+			const int s = min(s0 + j, Tn - 1), sn = min(s0 + j + 1, Tn - 1);
+			float a = 0.0f, dp = 0.0f;
+			fused_pipe_chunks<W, 0, FUSED_DA>(qr, gr, a, dp, unused, scale, b0l, b0h, b1l, b1h, kb + s * row, vb + s * row,
+			                                  kb + sn * row);
+			tile[j][lane * PH + wave] = expf(a * scale - l) * (dp - S);
+		}
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < DA_SJ; j++)
+			if (o_ok && s0 + j < Tn) o_base[(int64_t)(s0 + j) * pitch] = tile[j][o_t * PH + o_h];
+		__syncthreads();
+	}
+	swait32(b0l, b0h);  // drain the last prefetch before the wave ends
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void fused_bwd_dv_pipe(const float* __restrict__ dvo, const float* __restrict__ q,
+                                                           const float* __restrict__ k, const float* __restrict__ lse,
+                                                           float* __restrict__ dv, int Tn, int H, int n_hg, int NH,
+                                                           float scale)
+{
+	static_assert(W % 32 == 0, "whole 32-float chunks");
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const LogicalBlock lb = xcd_remap();
+	const int b = lb.y / n_hg, hg = lb.y % n_hg;
+	const int h_raw = hg * NH + wave;
+	const int h = min(h_raw, H - 1);
+	const int s_raw = lb.x * 64 + lane;
+	const int s = min(s_raw, Tn - 1);
+	const bool store = h_raw < H && s_raw < Tn;
+
+	float kr[W], acc[W];
+	{
+		const float4* kp = reinterpret_cast<const float4*>(k + (((int64_t)b * Tn + s) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++) {
+			const float4 x = kp[w4];
+			kr[w4 * 4 + 0] = x.x; kr[w4 * 4 + 1] = x.y; kr[w4 * 4 + 2] = x.z; kr[w4 * 4 + 3] = x.w;
+		}
+#pragma unroll
+		for (int w = 0; w < W; w++) acc[w] = 0.0f;
+#pragma unroll
+		for (int w = 0; w < W; w++) asm volatile("" : "+v"(kr[w]));
+	}
+	const int64_t row = (int64_t)H * W;
+	const float* const qb = q + (((int64_t)b * Tn) * H + h) * (int64_t)W;    // dst token 0 of this (b,h): wave-uniform
+	const float* const gb = dvo + (((int64_t)b * Tn) * H + h) * (int64_t)W;
+	const float* const lp = lse + ((int64_t)b * Tn) * H + h;
+	float unused = 0.0f;
+	float l = lp[0];
+	sarrived(l);  // before the first prefetch is issued
+	f32x16 b0l, b0h, b1l, b1h;
+	sload32(b0l, b0h, qb);
+	__builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+	for (int t = 0; t < Tn; t++) {
+		const int tn = min(t + 1, Tn - 1);
+		float l_next = lp[(int64_t)tn * H];  // issued here, taken inside right after the first chunk's wait
+		float a = 0.0f, p = 0.0f;
+		fused_pipe_chunks<W, 0, FUSED_DV>(kr, acc, a, p, unused, scale, b0l, b0h, b1l, b1h, qb + t * row, gb + t * row,
+		                                  qb + tn * row, l, &l_next);
+		l = l_next;
+	}
+	swait32(b0l, b0h);  // drain the last prefetch before the wave ends
+	if (store) {
+		float4* op = reinterpret_cast<float4*>(dv + (((int64_t)b * Tn + s) * H + h) * (int64_t)W);
+#pragma unroll
+		for (int w4 = 0; w4 < W / 4; w4++)
+			op[w4] = make_float4(acc[w4 * 4 + 0], acc[w4 * 4 + 1], acc[w4 * 4 + 2], acc[w4 * 4 + 3]);
+	}
+}
+
 bool shape_ok(int64_t B, int64_t T, int64_t H, int64_t W, int64_t Wv)
 {
 	return B >= 0 && T >= 0 && H >= 0 && W >= 1 && Wv >= 1;
@@ -499,9 +651,11 @@ int l1attn_fused_fwd_f64(const double* q, const double* k, const double* v, doub
 
 // First stage of the fused backward: dA [B,S,T,H] (gradient of the logits) and dv from dvo and the forward's
 // vo and lse.  dq and dk follow from l1attn_dense_bwd_* on dA, q, k.
-int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k, const float* v, const float* vo,
+// pipe: take the software-pipelined kernels where they exist (W == Wv in {32, 64}); every other shape runs what
+// l1attn_fused_bwd_stage_f32 runs
+static int fused_bwd_stage_f32(const float* dvo, const float* q, const float* k, const float* v, const float* vo,
                                const float* lse, float* dA, float* dv, int64_t B, int64_t T, int64_t H, int64_t W,
-                               int64_t Wv, void* stream)
+                               int64_t Wv, void* stream, bool pipe)
 {
 	if (!shape_ok(B, T, H, W, Wv)) return L1ATTN_ERR_ARG;
 	if (B * T * H == 0) return L1ATTN_OK;
@@ -527,7 +681,16 @@ int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k,
 		hipLaunchKernelGGL(fused_bwd_dv_tile<WV>, grid, block, 0, st, dvo, q, k, lse, dv, (int)T, (int)H, (int)n_hg,  \
 		                   NH, scale);                                                                              \
 		break
-	switch (W) {
+#define L1_FUSED_BWD_PIPE_CASE(WV)                                                                                  \
+	do {                                                                                                            \
+		hipLaunchKernelGGL(fused_bwd_da_pipe<WV>, grida, blocka, 0, st, dvo, q, k, v, vo, lse, dA, (int)T, (int)H,   \
+		                   (int)n_hga, NHa, scale);                                                                 \
+		hipLaunchKernelGGL(fused_bwd_dv_pipe<WV>, grid, block, 0, st, dvo, q, k, lse, dv, (int)T, (int)H, (int)n_hg,  \
+		                   NH, scale);                                                                              \
+	} while (0)
+	if (pipe && W == 32) L1_FUSED_BWD_PIPE_CASE(32);
+	else if (pipe && W == 64) L1_FUSED_BWD_PIPE_CASE(64);
+	else switch (W) {
 		L1_FUSED_BWD_CASE(16);
 		L1_FUSED_BWD_CASE(32);
 		L1_FUSED_BWD_CASE(48);
@@ -536,8 +699,23 @@ int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k,
 	default: return L1ATTN_ERR_ARG;
 	}
 #undef L1_FUSED_BWD_CASE
+#undef L1_FUSED_BWD_PIPE_CASE
 	L1_LAUNCH_CHECK();
 	return L1ATTN_OK;
+}
+
+int l1attn_fused_bwd_stage_f32(const float* dvo, const float* q, const float* k, const float* v, const float* vo,
+                               const float* lse, float* dA, float* dv, int64_t B, int64_t T, int64_t H, int64_t W,
+                               int64_t Wv, void* stream)
+{
+	return fused_bwd_stage_f32(dvo, q, k, v, vo, lse, dA, dv, B, T, H, W, Wv, stream, false);
+}
+
+int l1attn_fused_bwd_stage_pipe_f32(const float* dvo, const float* q, const float* k, const float* v, const float* vo,
+                                    const float* lse, float* dA, float* dv, int64_t B, int64_t T, int64_t H, int64_t W,
+                                    int64_t Wv, void* stream)
+{
+	return fused_bwd_stage_f32(dvo, q, k, v, vo, lse, dA, dv, B, T, H, W, Wv, stream, true);
 }
 
 int l1attn_fused_bwd_stage_f64(const double* dvo, const double* q, const double* k, const double* v, const double* vo,

@@ -33,5 +33,13 @@ __device__ __forceinline__ void swait32(f32x16& lo, f32x16& hi)
 {
 	asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(lo), "+s"(hi));
 }
+// A wave-uniform value that the compiler loads itself (an ordinary scalar load it tracks) is taken here: the
+// compiler puts its wait for that load in front of this point.  Placed right after a swait32, where nothing is in
+// flight, that wait costs nothing; left to the first use, it would fall between a prefetch and the work that
+// covers it, and wait for the prefetch as well.
+__device__ __forceinline__ void sarrived(float& x)
+{
+	asm volatile("" : "+s"(x));
+}
 
 #endif

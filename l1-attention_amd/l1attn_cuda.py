@@ -48,22 +48,27 @@ class L1AttnFusedFn(Function):
     example-setfind/setfind.py:128-136.  The reference has no such function (README.md:21 asks for it).
     The backward holds one [B,T,T,H] tensor (the gradient of the logits) where the composition holds four."""
     @staticmethod
-    def forward(ctx, q, k, v):
+    def forward(ctx, q, k, v, *pipelined):
+        # apply(q, k, v) or apply(q, k, v, pipelined): the flag picks the software-pipelined kernels (same results)
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        vo, lse = _drv.dense_fused_forward(q, k, v, want_lse=True)
+        ctx.pipelined, ctx.n_flags = bool(pipelined and pipelined[0]), len(pipelined)
+        vo, lse = _drv.dense_fused_forward(q, k, v, want_lse=True, pipelined=ctx.pipelined)
         ctx.save_for_backward(q, k, v, vo, lse)
         return vo
 
     @staticmethod
     def backward(ctx, d_vo):
         q, k, v, vo, lse = ctx.saved_tensors[:5]
-        d_q, d_k, d_v = _drv.dense_fused_backward(d_vo.contiguous(), q, k, v, vo, lse)
-        return d_q, d_k, d_v
+        d_q, d_k, d_v = _drv.dense_fused_backward(d_vo.contiguous(), q, k, v, vo, lse, pipelined=ctx.pipelined)
+        return (d_q, d_k, d_v) + (None,) * ctx.n_flags
 
 
 class L1AttnFused(nn.Module):
-    def __init__(self):
+    """pipelined: the kernels that stream the wave-uniform rows through a software pipeline of scalar loads, where
+    they exist (float32, widths 32 and 64); same results bit for bit."""
+    def __init__(self, pipelined=False):
         super(L1AttnFused, self).__init__()
+        self.pipelined = bool(pipelined)
 
     def forward(self, q, k, v):
-        return L1AttnFusedFn.apply(q, k, v)
+        return L1AttnFusedFn.apply(q, k, v, self.pipelined)

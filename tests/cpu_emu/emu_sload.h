@@ -39,4 +39,5 @@ static inline void swait32(f32x16&, f32x16&)
 	}
 	emu_sload::pending.clear();
 }
+static inline void sarrived(float&) {}
 static inline void __builtin_amdgcn_sched_barrier(int) {}

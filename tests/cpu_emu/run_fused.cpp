@@ -1,6 +1,6 @@
 // TEST INFRASTRUCTURE: runs l1attn_fused_fwd_f32 / _f64 of csrc/fused.hip, compiled for the host with
 // the stand-in header next to this file, on inputs read from a file, and writes vo and lse.
-//   run_fused <in> <out> <f32|f64> <misalign> [pipe]      (pipe: forward through l1attn_fused_fwd_pipe_f32)
+//   run_fused <in> <out> <f32|f64> <misalign> [pipe]      (pipe: l1attn_fused_fwd_pipe_f32 and l1attn_fused_bwd_stage_pipe_f32)
 // in : int64 B,T,H,W,Wv then q,k [B,T,H,W], v [B,T,H,Wv] and dvo [B,T,H,Wv] in the chosen type
 // out: vo [B,T,H,Wv], lse [B,T,H], one int64 (threads the forward ran), then the backward's first stage on
 //      the forward's own vo and lse: dA [B,T,T,H], dv [B,T,H,Wv], one int64 (threads it ran)
@@ -41,13 +41,17 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, bool f32, int mis, bool pip
 	T *dvo = alloc(nv), *dA = alloc(na), *dv = alloc(nv);
 	if (fread(dvo, sizeof(T), nv, fi) != nv) return 3;
 	emu::n_threads_run = 0;
-	if (f32) rc = l1attn_fused_bwd_stage_f32((const float*)dvo, (const float*)q, (const float*)k, (const float*)v,
+	if (f32 && pipe) rc = l1attn_fused_bwd_stage_pipe_f32((const float*)dvo, (const float*)q, (const float*)k, (const float*)v,
+	                                                      (const float*)vo, (const float*)lse, (float*)dA, (float*)dv, B, Tn,
+	                                                      H, W, Wv, nullptr);
+	else if (f32) rc = l1attn_fused_bwd_stage_f32((const float*)dvo, (const float*)q, (const float*)k, (const float*)v,
 	                                         (const float*)vo, (const float*)lse, (float*)dA, (float*)dv, B, Tn, H, W,
 	                                         Wv, nullptr);
 	else rc = l1attn_fused_bwd_stage_f64((const double*)dvo, (const double*)q, (const double*)k, (const double*)v,
 	                                     (const double*)vo, (const double*)lse, (double*)dA, (double*)dv, B, Tn, H, W,
 	                                     Wv, nullptr);
 	if (rc) return 20 + (rc < 0 ? -rc : rc);
+	if (emu_sload::outstanding != 0) return 9;
 	fwrite(dA, sizeof(T), na, fo);
 	fwrite(dv, sizeof(T), nv, fo);
 	n = emu::n_threads_run;

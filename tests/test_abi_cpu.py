@@ -430,6 +430,12 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
         drv.dense_fused_forward(q, k, v.double())
     grads = drv.dense_fused_backward(torch.zeros_like(v), q, k, v, vo, lse)
     assert [g.shape for g in grads] == [q.shape, k.shape, v.shape]
+    assert "l1attn_fused_bwd_stage_f32" in _FakeLib.calls and "l1attn_fused_bwd_stage_pipe_f32" not in _FakeLib.calls
+    drv.dense_fused_backward(torch.zeros_like(v), q, k, v, vo, lse, pipelined=True)
+    assert "l1attn_fused_bwd_stage_pipe_f32" in _FakeLib.calls
+    drv.dense_fused_backward(torch.zeros_like(v).double(), q.double(), k.double(), v.double(), vo.double(), lse.double(),
+                             pipelined=True)                                          # float64 has one entry
+    assert _FakeLib.calls[-1].startswith("l1attn_dense_bwd") and "l1attn_fused_bwd_stage_f64" in _FakeLib.calls
     with pytest.raises(RuntimeError, match="lse must be"):
         drv.dense_fused_backward(torch.zeros_like(v), q, k, v, vo, lse[:, :-1])
     with pytest.raises(RuntimeError, match="dvo must have"):

@@ -107,7 +107,7 @@ def test_extra_legs(bench, monkeypatch, capsys):
     x = out["extra"]
     assert set(x) == {"fused_forward", "sparse_16bit", "fixed_point_forward", "instruction_rates", "column_ranks_B2_T48_H2_W32"}
     for row in x["fused_forward"].values():
-        assert row["max_rel_diff"] < 1e-5 and set(row["fwd_bwd"]) == {"fused", "composed"}
+        assert row["max_rel_diff"] < 1e-5 and set(row["fwd_bwd"]) == {"fused", "fused_pipelined", "composed"}
     for row in x["sparse_16bit"].values():
         assert all(row[dt + leg] > 0 for dt in ("float32", "float16", "bfloat16") for leg in ("_fwd_ms", "_fwd_bwd_ms"))
     assert len(x["instruction_rates"]) == 4

@@ -120,7 +120,8 @@ def test_fused_tiled_kernels_on_cpu(runner, tmp_path, shape):
 
 @pytest.mark.parametrize("shape", [(2, 64, 4, 32), (1, 100, 3, 64), (2, 70, 6, 32), (1, 33, 9, 64), (1, 1000, 1, 32)])
 def test_fused_pipelined_forward_on_cpu(runner, tmp_path, shape):
-    """The software-pipelined forward (l1attn_fused_fwd_pipe_f32).  The host stand-in for the scalar prefetch
+    """The software-pipelined forward (l1attn_fused_fwd_pipe_f32) and, in the same run, the pipelined first stage of
+    the backward (l1attn_fused_bwd_stage_pipe_f32: dA and dv).  The host stand-in for the scalar prefetch
     delivers a chunk's data at the wait and poisons the buffer at the load, so reading a buffer before its wait, a
     chunk taken from the wrong buffer, a wrong chunk address or a missing final drain all fail here.  Same arithmetic
     in the same order as the plain tiled kernel: equal bit for bit."""
@@ -132,8 +133,12 @@ def test_fused_pipelined_forward_on_cpu(runner, tmp_path, shape):
     NH = min(H, 4)
     assert piped["threads"] == -(-T // 64) * B * -(-H // NH) * 64 * NH
     assert torch.equal(piped["vo"], plain["vo"]) and torch.equal(piped["lse"], plain["lse"])
+    assert torch.equal(piped["dA"], plain["dA"]) and torch.equal(piped["dv"], plain["dv"])
+    NHa = min(H, 8)  # the dA kernel takes up to eight heads per workgroup
+    assert piped["bwd_threads"] == plain["bwd_threads"] == -(-T // 64) * B * (-(-H // NHa) * 64 * NHa + -(-H // NH) * 64 * NH)
     ref, ref_lse = _ref(q, k, v)
     assert cf.rel_err(piped["vo"], ref) <= 1e-5 and cf.rel_err(piped["lse"], ref_lse) <= 1e-5
+    _check_backward(piped, q, k, v, 1e-4)
     # widths without a pipelined kernel run what the plain entry runs
     if shape == (2, 64, 4, 32):
         q16, k16, v16 = q[..., :16].contiguous(), k[..., :16].contiguous(), v[..., :16].contiguous()
@@ -183,6 +188,9 @@ def test_fused_kernels_have_no_data_race_between_barriers(runner_tsan, tmp_path)
     q, k, v = (torch.randn(B, T, H, W, generator=g) for _ in range(3))
     r = _run(runner_tsan, tmp_path, q, k, v)
     _check_backward(r, q, k, v, 1e-4)
+    # the pipelined dA kernel keeps a scalar prefetch in flight across the flush and its two barriers
+    q, k, v = (torch.randn(1, 70, 9, 32, generator=g) for _ in range(3))
+    _check_backward(_run(runner_tsan, tmp_path, q, k, v, pipe=True), q, k, v, 1e-4)
 
 
 def test_fixed_point_prepass_kernels_on_cpu(tmp_path):

@@ -271,7 +271,7 @@ def test_launch_geometry_at_full_size(runner):
     assert launches[:4] == [("dense_fwd_f32_pipe<64, false>", (64, 4, 8), 1024, 0),
                             ("dense_bwd_f32_fast<64, 512, 4, true, true, true>", (16, 2, 8), 512, 4 * 8 * 68 * 4),
                             ("dense_bwd_reduce_colsum", (2048, 1, 1), 256, 0),
-                            ("dense_bwd_reduce_dk<true, true>", (32768, 1, 1), 256, 0)]
+                            ("dense_bwd_reduce_dk<true, true, false>", (32768, 1, 1), 256, 0)]
     rcs, launches = _dims(runner, (16, 1024, 8, 64))
     assert rcs["backward"] == "0" and launches[1] == ("dense_bwd_f32_fast<64, 512, 4, false, false, true>", (16, 1, 16), 512, 8704)
     assert _dims(runner, (2, 64, 4, 32))[0]["backward"] == "0"

@@ -61,7 +61,7 @@ def cpu_stand_ins(monkeypatch):
         esum = e.sum(1)
         return [torch.einsum("bsdh,bshw->bdhw", e / (1.0 + esum)[:, None], v), torch.log1p(esum) if want_lse else None]
 
-    def fused_bwd(dvo, q, k, v, vo, lse):
+    def fused_bwd(dvo, q, k, v, vo, lse, pipelined=False):
         with torch.enable_grad():  # (called from inside a Function's backward, where recording is off)
             leaves = [x.detach().clone().requires_grad_() for x in (q, k, v)]
             return list(torch.autograd.grad(cf.dense_then_value(*leaves, noop=True), leaves, dvo))
@@ -108,6 +108,8 @@ def test_wip_fused_gpu_tests_walk_on_stand_ins(cpu_stand_ins):
         t.test_fused_forward_vs_oracle(shape)
     for shape in [(2, 64, 4, 32), (1, 100, 3, 64), (1, 40, 2, 48)]:
         t.test_fused_pipelined_forward_equals_the_plain_one(shape)
+    for shape in [(2, 64, 4, 32), (1, 33, 9, 64)]:
+        t.test_fused_pipelined_backward_stage_equals_the_plain_one(shape)
     t.test_fused_forward_unaligned_views_take_the_generic_kernel()
     for shape in t.BWD_SHAPES:
         t.test_fused_backward_vs_oracle(shape)

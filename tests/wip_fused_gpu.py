@@ -96,6 +96,26 @@ def test_fused_pipelined_forward_equals_the_plain_one(shape):
         assert cf.rel_err(vop.cpu(), ref) <= F32_TOL and cf.rel_err(lsep.cpu(), ref_lse) <= F32_TOL
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 4, 32), (1, 100, 3, 64), (2, 70, 9, 32), (1, 33, 9, 64), (2, 512, 8, 64)])
+def test_fused_pipelined_backward_stage_equals_the_plain_one(shape):
+    """l1attn_fused_bwd_stage_pipe_f32 (the dA and dv kernels with their wave-uniform rows through the scalar-load
+    pipeline; widths 32 and 64): the same arithmetic in the same order, so dq, dk and dv of the whole backward
+    equal the plain route's bit for bit.  Run after the plain backward's tests have passed."""
+    B, T, H, W = shape
+    print("case fused pipelined backward", shape, flush=True)
+    import _l1attn_hip as drv
+    g = torch.Generator().manual_seed(sum(shape) + 3)
+    q, k, v, dvo = (torch.randn(B, T, H, W, generator=g).cuda() for _ in range(4))
+    vo, lse = drv.dense_fused_forward(q, k, v, want_lse=True)
+    plain = drv.dense_fused_backward(dvo, q, k, v, vo, lse)
+    piped = drv.dense_fused_backward(dvo, q, k, v, vo, lse, pipelined=True)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(piped, plain))
+    x = [t.clone().requires_grad_() for t in (q, k, v)]
+    via_module = torch.autograd.grad(_fused().L1AttnFused(pipelined=True)(*x), x, dvo)
+    assert all(torch.equal(a, b) for a, b in zip(via_module, plain))
+
+
 def test_fused_forward_unaligned_views_take_the_generic_kernel():
     print("case fused unaligned", flush=True)
     import _l1attn_hip as drv
