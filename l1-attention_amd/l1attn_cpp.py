@@ -53,7 +53,9 @@ class L1AttnFusedFn(Function):
 
 
 class L1AttnFused(nn.Module):
-    def __init__(self):
+    """pipelined: accepted for symmetry with l1attn_cuda.L1AttnFused (a choice between GPU kernels with equal
+    results); it has no meaning on the host."""
+    def __init__(self, pipelined=False):
         super(L1AttnFused, self).__init__()
 
     def forward(self, q, k, v):
