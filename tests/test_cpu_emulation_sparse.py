@@ -105,10 +105,11 @@ TOL = {"f16": 2.0 ** -10, "bf16": 2.0 ** -7}
 TORCH_T = {"f16": torch.float16, "bf16": torch.bfloat16}
 
 
-@pytest.mark.parametrize("shape", [(2, 9, 3, 5, 5, 40),      # scalar path, dst rows without edges
-                                   (1, 24, 8, 32, 32, 150),   # configuration-4 head geometry, 8-byte pieces
-                                   (1, 20, 3, 8, 12, 90)])    # value width differs from key width
-@pytest.mark.parametrize("sm", [True, False])
+@pytest.mark.parametrize("shape,sm", [((2, 9, 3, 5, 5, 40), True),       # scalar path, dst rows without edges
+                                      ((2, 9, 3, 5, 5, 40), False),
+                                      ((1, 24, 8, 32, 32, 150), True),   # configuration-4 head geometry, 8-byte pieces
+                                      ((1, 20, 3, 8, 12, 90), True),     # value width differs from key width
+                                      ((1, 20, 3, 8, 12, 90), False)])
 def test_sparse_forward_kernels_on_cpu(runner, tmp_path, shape, sm):
     B, T, H, W, Wv, E = shape
     g = torch.Generator().manual_seed(sum(shape))

@@ -1,0 +1,125 @@
+"""CPU-only: the GPU test files run end to end on the CPU -- the real Python operators and drivers, the real ctypes
+binding with its argtypes, and a library built from the product's kernel sources for the host
+(tests/cpu_emu/lib_*.cpp: dense.hip, fixed.hip, fused.hip, rank_sort.hip and sparse.hip as they are, GPU threads as OS
+threads; host stand-ins only for coo.hip and the library sort, whose kernels cannot run that way).
+
+Everything else on the CPU either runs the kernels through C++ runners (which call the entry points themselves) or
+walks the drivers against stand-ins that accept anything.  Neither notices a driver that passes the right kinds of
+arguments in the wrong order.  Here the drivers' own calls reach the kernels, and the GPU tests' own comparisons
+against the oracle judge the result: the test functions are taken from tests/test_*_gpu.py and tests/wip_*_gpu.py
+unchanged, at the shapes an emulation can walk.  Tensors stay on the CPU: `.cuda()` is a copy in host memory and
+`Tensor.is_cuda` says yes."""
+import contextlib
+import ctypes
+import importlib.util
+import os
+import subprocess
+
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+EMU = os.path.join(HERE, "cpu_emu")
+CLANG = "/opt/rocm/llvm/bin/clang++"
+PARTS = (("lib_dense", "g++"), ("lib_fixed", "g++"), ("lib_fused", "g++"), ("lib_ranks", "g++"), ("lib_sparse", CLANG),
+         ("lib_host", "g++"))
+
+pytestmark = pytest.mark.skipif(not os.path.exists(CLANG), reason="needs ROCm's clang++ (bfloat16 and float16 on the host)")
+
+
+@pytest.fixture(scope="module")
+def emulated_library_path(tmp_path_factory):
+    d = tmp_path_factory.mktemp("emulib")
+    jobs = []
+    for name, cxx in PARTS:
+        lines = "-gline-tables-only" if cxx == CLANG else "-g1"
+        cmd = [cxx, "-std=c++20", "-O1", lines, "-fPIC", "-pthread", "-I", EMU, "-x", "c++", "-c",
+               os.path.join(EMU, name + ".cpp"), "-o", str(d / (name + ".o"))]
+        jobs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for cmd, p in jobs:
+        text, _ = p.communicate()
+        assert p.returncode == 0, "%s\n%s" % (" ".join(cmd), text[-3000:])
+    lib = str(d / "libl1attn_emu.so")
+    # linked by clang++: its runtime holds the float <-> bfloat16 conversions the sparse kernels call on the host
+    subprocess.run([CLANG, "-shared", "-pthread", "-o", lib] + [str(d / (n + ".o")) for n, _ in PARTS], check=True)
+    return lib
+
+
+@pytest.fixture()
+def on_the_emulated_library(emulated_library_path, monkeypatch):
+    import _l1attn_hip as drv
+    monkeypatch.setattr(drv, "_LIB_PATH", emulated_library_path)
+    monkeypatch.setattr(drv, "_lib", None)                 # lib() loads the path above and sets its argtypes on it
+    monkeypatch.setattr(drv, "_enabled", set(drv.EXPERIMENTAL))
+    monkeypatch.setattr(drv, "stream_of", lambda x: ctypes.c_void_p(None))
+    # a copy, as on a GPU: x.cuda().requires_grad_() must not turn x itself into a leaf that collects gradients
+    monkeypatch.setattr(torch.Tensor, "cuda", lambda self, *a, **k: self.clone())
+    real_to = torch.Tensor.to
+
+    def to(self, *a, **k):  # .to("cuda") stays where it is
+        is_gpu = lambda x: (isinstance(x, str) and x.startswith("cuda")) or (isinstance(x, torch.device) and x.type == "cuda")
+        a = tuple("cpu" if is_gpu(x) else x for x in a)
+        if is_gpu(k.get("device")):
+            k["device"] = "cpu"
+        return real_to(self, *a, **k)
+
+    monkeypatch.setattr(torch.Tensor, "to", to)
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda *a, **k: None)
+    monkeypatch.setattr(torch.cuda, "device", lambda d: contextlib.nullcontext())
+    assert drv.lib().l1attn_version() == -1                # the emulated library, not the product's
+    return drv
+
+
+def _load(name):
+    spec = importlib.util.spec_from_file_location(name, os.path.join(HERE, name + ".py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_dense_gpu_tests_on_the_emulated_library(on_the_emulated_library):
+    t = _load("test_dense_gpu")
+    for shape in [(2, 64, 4, 32), (2, 3, 16, 7), (1, 100, 3, 33), (1, 40, 2, 128), (3, 33, 1, 65)]:
+        t.test_dense_f32_vs_oracle(shape)
+    for shape in [(1, 16, 8, 64), (2, 5, 3, 7)]:
+        t.test_dense_f64_vs_oracle(shape)
+    t.test_dense_golden_reference_extension()
+    t.test_dense_ties_onehot_fixture()
+    t.test_dense_deterministic_and_inputs_untouched()
+    t.test_dense_forward_odd_width_with_and_without_workspace()
+    t.test_dense_in_a_model_block()
+
+
+def test_sparse_gpu_tests_on_the_emulated_library(on_the_emulated_library):
+    t = _load("test_sparse_gpu")
+    t.test_check_sparse_cases_vs_oracle(torch.float64, True)       # full, permuted, permuted minus four; uni and bidi
+    t.test_sparse_and_bidi_f32_vs_oracle(t.SHAPES[0], False)
+    t.test_sparse_golden_reference_extension("sA", True)
+    t.test_sparse_full_list_equals_dense_attention(False)         # sparse operator against the dense operator
+    t.test_sparse_value_width_differs_from_key_width()
+
+
+def test_fused_gpu_tests_on_the_emulated_library(on_the_emulated_library):
+    t = _load("wip_fused_gpu")
+    for shape in t.SHAPES[:2] + t.SHAPES[4:5] + t.SHAPES[8:9]:
+        t.test_fused_forward_vs_oracle(shape)
+    for shape in [(2, 64, 4, 32), (1, 40, 2, 48)]:
+        t.test_fused_pipelined_forward_equals_the_plain_one(shape)
+    t.test_fused_pipelined_backward_stage_equals_the_plain_one((1, 33, 9, 64))
+    for shape in t.BWD_SHAPES[:2]:
+        t.test_fused_backward_vs_oracle(shape)
+    t.test_fused_backward_in_batch_slabs_equals_the_whole_batch()
+    t.test_fused_gradcheck_fp64()
+    t.test_fused_in_a_model_block(21)
+    t.test_fixed_point_forward_vs_oracle((2, 64, 4, 32), False)
+
+
+def test_sparse_half_gpu_tests_on_the_emulated_library(on_the_emulated_library):
+    t = _load("wip_sparse_half_gpu")
+    t.test_half_forward_vs_f32_entry_and_oracle(torch.float16, t.SHAPES[0], True)
+    t.test_half_forward_vs_f32_entry_and_oracle(torch.bfloat16, t.SHAPES[1], False)
+    t.test_half_backward_vs_autograd_closed_form(torch.float16, (2, 20, 3, 8, 12, 90), False)
+    t.test_half_backward_vs_autograd_closed_form(torch.bfloat16, (2, 9, 3, 5, 5, 40), True)
+    for dt in t.DTYPES:
+        t.test_half_empty_list(dt)
