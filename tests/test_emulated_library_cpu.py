@@ -78,48 +78,65 @@ def _load(name):
     return mod
 
 
+# One or two small cases per driver function: what this file adds to the other CPU tests is that every pointer and
+# size a driver passes lands in the right parameter; the kernels' shapes are walked in tests/test_cpu_emulation*.py.
+# L1ATTN_EMULATED_LIBRARY_FULL=1 runs the longer selection (about four minutes).
+FULL = bool(os.environ.get("L1ATTN_EMULATED_LIBRARY_FULL"))
+
+
 def test_dense_gpu_tests_on_the_emulated_library(on_the_emulated_library):
     t = _load("test_dense_gpu")
-    for shape in [(2, 64, 4, 32), (2, 3, 16, 7), (1, 100, 3, 33), (1, 40, 2, 128), (3, 33, 1, 65)]:
+    shapes = [(2, 64, 4, 32), (2, 3, 16, 7), (1, 100, 3, 33)]
+    if FULL:
+        shapes += [(1, 16, 8, 64), (1, 70, 20, 48), (1, 40, 2, 128), (3, 33, 1, 65)]
+    for shape in shapes:
         t.test_dense_f32_vs_oracle(shape)
-    for shape in [(1, 16, 8, 64), (2, 5, 3, 7)]:
+    for shape in [(2, 5, 3, 7)] + ([(2, 64, 4, 32), (1, 16, 8, 64), (1, 100, 3, 33)] if FULL else []):
         t.test_dense_f64_vs_oracle(shape)
     t.test_dense_golden_reference_extension()
-    t.test_dense_ties_onehot_fixture()
-    t.test_dense_deterministic_and_inputs_untouched()
     t.test_dense_forward_odd_width_with_and_without_workspace()
     t.test_dense_in_a_model_block()
+    if FULL:
+        t.test_dense_ties_onehot_fixture()
+        t.test_dense_deterministic_and_inputs_untouched()
 
 
 def test_sparse_gpu_tests_on_the_emulated_library(on_the_emulated_library):
     t = _load("test_sparse_gpu")
     t.test_check_sparse_cases_vs_oracle(torch.float64, True)       # full, permuted, permuted minus four; uni and bidi
-    t.test_sparse_and_bidi_f32_vs_oracle(t.SHAPES[0], False)
     t.test_sparse_golden_reference_extension("sA", True)
-    t.test_sparse_full_list_equals_dense_attention(False)         # sparse operator against the dense operator
     t.test_sparse_value_width_differs_from_key_width()
+    if FULL:
+        t.test_check_sparse_cases_vs_oracle(torch.float32, False)
+        for shape in t.SHAPES[:4]:
+            for sm in (True, False):
+                t.test_sparse_and_bidi_f32_vs_oracle(shape, sm)
+        t.test_sparse_golden_reference_extension("sB", False)
+        t.test_sparse_full_list_equals_dense_attention(False)     # sparse operator against the dense operator
 
 
 def test_fused_gpu_tests_on_the_emulated_library(on_the_emulated_library):
     t = _load("wip_fused_gpu")
-    for shape in t.SHAPES[:2] + t.SHAPES[4:5] + t.SHAPES[8:9]:
+    for shape in (t.SHAPES if FULL else t.SHAPES[:1] + t.SHAPES[4:5] + t.SHAPES[8:9]):
         t.test_fused_forward_vs_oracle(shape)
-    for shape in [(2, 64, 4, 32), (1, 40, 2, 48)]:
+    for shape in [(2, 64, 4, 32)] + ([(1, 100, 3, 64), (1, 33, 9, 64), (1, 40, 2, 48)] if FULL else []):
         t.test_fused_pipelined_forward_equals_the_plain_one(shape)
     t.test_fused_pipelined_backward_stage_equals_the_plain_one((1, 33, 9, 64))
-    for shape in t.BWD_SHAPES[:2]:
+    for shape in (t.BWD_SHAPES[:5] if FULL else t.BWD_SHAPES[:1]):
         t.test_fused_backward_vs_oracle(shape)
     t.test_fused_backward_in_batch_slabs_equals_the_whole_batch()
-    t.test_fused_gradcheck_fp64()
-    t.test_fused_in_a_model_block(21)
     t.test_fixed_point_forward_vs_oracle((2, 64, 4, 32), False)
+    if FULL:
+        t.test_fused_gradcheck_fp64()
+        t.test_fused_in_a_model_block(21)
 
 
 def test_sparse_half_gpu_tests_on_the_emulated_library(on_the_emulated_library):
     t = _load("wip_sparse_half_gpu")
     t.test_half_forward_vs_f32_entry_and_oracle(torch.float16, t.SHAPES[0], True)
-    t.test_half_forward_vs_f32_entry_and_oracle(torch.bfloat16, t.SHAPES[1], False)
-    t.test_half_backward_vs_autograd_closed_form(torch.float16, (2, 20, 3, 8, 12, 90), False)
     t.test_half_backward_vs_autograd_closed_form(torch.bfloat16, (2, 9, 3, 5, 5, 40), True)
     for dt in t.DTYPES:
         t.test_half_empty_list(dt)
+    if FULL:
+        t.test_half_forward_vs_f32_entry_and_oracle(torch.bfloat16, t.SHAPES[1], False)
+        t.test_half_backward_vs_autograd_closed_form(torch.float16, (2, 20, 3, 8, 12, 90), False)
