@@ -140,3 +140,60 @@ def test_sparse_half_gpu_tests_on_the_emulated_library(on_the_emulated_library):
     if FULL:
         t.test_half_forward_vs_f32_entry_and_oracle(torch.bfloat16, t.SHAPES[1], False)
         t.test_half_backward_vs_autograd_closed_form(torch.float16, (2, 20, 3, 8, 12, 90), False)
+
+
+def test_bench_on_the_emulated_library(on_the_emulated_library, monkeypatch, capsys):
+    """bench.py's default run and its --extra legs at shrunken sizes, with the real drivers and kernels behind
+    them: the script's own direct library calls (instruction probes, both column-rank entry points) and every leg's
+    value check run for real.  Timings mean nothing here."""
+    import json
+    import sys
+    import time
+
+    import bench as b
+
+    class Event(object):
+        def __init__(self, enable_timing=False):
+            self.t = None
+
+        def record(self, stream=None):
+            self.t = time.perf_counter()
+
+        def elapsed_time(self, other):
+            return max((other.t - self.t) * 1e3, 1e-6)
+
+    def once(fn, iters, warm=2):  # time_gpu with a single call: an emulated launch takes long enough
+        t0 = time.perf_counter()
+        fn()
+        return (time.perf_counter() - t0) * 1e3
+
+    monkeypatch.setattr(b, "time_gpu", once)
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    monkeypatch.setattr(torch.cuda, "Event", Event)
+    for name in ("empty_cache", "reset_peak_memory_stats"):
+        monkeypatch.setattr(torch.cuda, name, lambda *a, **k: None)
+    for name in ("memory_allocated", "max_memory_allocated"):
+        monkeypatch.setattr(torch.cuda, name, lambda *a, **k: 0)
+    monkeypatch.setattr(b, "DEVICE", "cpu")
+    monkeypatch.setattr(b, "HEADLINE", (1, 64, 1, 32))
+    monkeypatch.setattr(b, "SECOND", (1, 32, 1, 64))
+    monkeypatch.setattr(b, "CONFIG4", ((1, 24, 1, 32), 4))
+    monkeypatch.setattr(b, "CONFIG5", (1, 32, 1, 64))
+
+    def run(*argv):
+        monkeypatch.setattr(sys, "argv", ["bench.py"] + list(argv))
+        capsys.readouterr()
+        b.main()
+        return json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+
+    if FULL:
+        out = run("--steps", "1", "--warmup", "0", "--skip-cpu")
+        assert out["value"] > 0 and "error" not in out["sparse"] and "error" not in out["valu_probe"]
+        assert out["sparse"]["config4_uni"]["edges"] > 0 and out["sparse"]["config5_bidi"]["edges"] > 0
+        assert out["dense"]["backward_plan"]["step_loop_form"] == 0
+    x = run("--extra")["extra"]
+    for row in x["fused_forward"].values():
+        assert row["max_rel_diff"] < 1e-5                      # fused against the composition, both on the kernels
+    for row in x["fixed_point_forward"].values():
+        assert row["max_rel_diff_to_fp32_kernel_batch0"] < 1e-5
+    assert len(x["instruction_rates"]) == 4 and len(x["sparse_16bit"]) == 2
