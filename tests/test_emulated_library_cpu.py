@@ -197,3 +197,12 @@ def test_bench_on_the_emulated_library(on_the_emulated_library, monkeypatch, cap
     for row in x["fixed_point_forward"].values():
         assert row["max_rel_diff_to_fp32_kernel_batch0"] < 1e-5
     assert len(x["instruction_rates"]) == 4 and len(x["sparse_16bit"]) == 2
+
+
+def test_smoke_on_the_emulated_library(on_the_emulated_library, monkeypatch, capsys):
+    """__graft_entry__.smoke() as it is: dense, expandCoo, sparse and bidirectional against the oracle."""
+    import __graft_entry__ as entry
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    monkeypatch.setattr(torch.cuda, "get_device_name", lambda *a: "host emulation")
+    entry.smoke()
+    assert "smoke ok" in capsys.readouterr().out
