@@ -206,3 +206,15 @@ def test_smoke_on_the_emulated_library(on_the_emulated_library, monkeypatch, cap
     monkeypatch.setattr(torch.cuda, "get_device_name", lambda *a: "host emulation")
     entry.smoke()
     assert "smoke ok" in capsys.readouterr().out
+
+
+def test_late_gpu_tests_on_the_emulated_library(on_the_emulated_library):
+    """tests/test_y_configs_gpu.py, the part that is small enough: the native-module stand-ins called the way the
+    reference's autograd Functions call them, the two model blocks, and (longer selection) the sign-domain test and
+    the training loop."""
+    t = _load("test_y_configs_gpu")
+    t.test_native_module_stand_ins_on_the_gpu()
+    t.test_model_blocks_on_the_gpu()
+    if FULL:
+        t.test_sign_domain_of_the_fast_float32_backward()
+        t.test_training_steps_on_the_gpu_operator_match_torch_autograd()
