@@ -113,15 +113,12 @@ def dense_headline(steps, warmup):
         "fwd_bwd_gops": 6 * N / (ms_per_step * 1e-3) / 1e9,
     }
     out["frac_of_valu_peak"] = out["fwd_bwd_gops"] / 1e3 / P_VALU_TOPS
-    # which forms of the backward this process ran (both are chosen from the environment, read once by the library)
-    import ctypes
+    # which forms of the backward this process ran (--bwd-form / --rank-sort; the default entry point without them)
     import _l1attn_hip as drv
-    info = (ctypes.c_int64 * 16)()
-    drv.lib().l1attn_dense_bwd_plan_info(B, T, H, W, info)
+    info = drv.dense_backward_plan(B, T, H, W)
     out["backward_plan"] = {"rank_form": int(info[2]), "branch_free": int(info[3]), "tiles_per_workgroup": int(info[9]),
                             "step_loop_form": int(info[14]),
-                            "L1ATTN_BWD_PREFETCH": os.environ.get("L1ATTN_BWD_PREFETCH"),
-                            "L1ATTN_RANK_SORT": os.environ.get("L1ATTN_RANK_SORT")}
+                            "rank_sort": "merge" if (info[2] and drv._dense_bwd_form[1]) else "radix"}
     del dA, q, k
     torch.cuda.empty_cache()
     return out
@@ -573,6 +570,10 @@ def main():
                     help="only run the reference's timing grid (benchmark.py:57-66), one JSON line per cell")
     ap.add_argument("--extra", action="store_true",
                     help="only time the fused forward and the 16-bit sparse forwards beside what they replace")
+    ap.add_argument("--bwd-form", type=int, choices=(0, 1, 2), default=0,
+                    help="A/B aid: step loop of the long-sequence dense backward (0 = the default entry point)")
+    ap.add_argument("--rank-sort", choices=("radix", "merge"), default="radix",
+                    help="A/B aid: sort behind the dense backward's column ranks (radix = the default entry point)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: only run three 1 GiB device-to-device copies, the known-size "
                          "kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -588,6 +589,10 @@ def main():
         sys.exit(3)
     import _l1attn_hip
     _l1attn_hip.lib()  # fail here, loudly, if the HIP library is not built
+    if args.bwd_form or args.rank_sort == "merge":
+        _l1attn_hip.enable_experimental(*([("bwd_pipe")] if args.bwd_form else []),
+                                        *([("rank_merge")] if args.rank_sort == "merge" else []))
+        _l1attn_hip.set_dense_backward_form(args.bwd_form, int(args.rank_sort == "merge"))
 
     if args.copy_calibration:
         src = torch.empty(COPY_FLOATS, dtype=torch.float32, device=DEVICE).normal_()

@@ -91,9 +91,8 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
  *   8 staged d_attn values per thread, step   9 dst tiles per workgroup
  *  10 workgroups along T (= partial arrays)  11 LDS bytes per workgroup
  *  12 workspace bytes per batch              13 batches per launch with the full workspace
- *  14 form of the branch-free step loop: 0, or with L1ATTN_BWD_PREFETCH=2 / =3 in the environment (read once per
- *     process) 1 = two steps of prefetch distance, 2 = the same with two LDS planes and one barrier per step;
- *     bit-identical results in all three
+ *  14 form of the branch-free step loop the plan runs: 0 (always, through l1attn_dense_bwd_plan_info), or the
+ *     loop_form given to l1attn_dense_bwd_plan_info_ex where the plan is branch-free
  *  15 reserved (0)
  * Returns 0, or a negative argument error.
  */
@@ -104,6 +103,22 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k, double* dq, double* dk,
                          int64_t B, int64_t T, int64_t H, int64_t W,
                          void* workspace, size_t workspace_bytes, void* stream);
+/*
+ * l1attn_dense_bwd_f32 with its two internal choices as arguments; l1attn_dense_bwd_f32 is this call with
+ * (0, 0).  The library reads no environment variable and keeps no state between calls: a caller that wants a
+ * non-default form says so here, per call.  Same workspace as l1attn_dense_bwd_f32.
+ *   loop_form  step loop of the branch-free long-sequence plans: 0 one step of prefetch distance, 1 two steps,
+ *              2 two steps with two LDS planes and one barrier per step.  Bit-identical results; other plans
+ *              ignore it (l1attn_dense_bwd_plan_info_ex reports in info[14] what a shape runs).
+ *   rank_sort  where the plan takes sign() from column ranks: 0 ranks from l1attn_dense_column_ranks_f32,
+ *              1 from l1attn_dense_column_ranks_merge_f32.  Identical ranks.
+ * Other values: L1ATTN_ERR_ARG.  No counterpart in the reference; the non-zero choices exist so that they can be
+ * timed against the default and are not reached by the Python operators unless the caller opts in by name.
+ */
+int l1attn_dense_bwd_plan_info_ex(int64_t B, int64_t T, int64_t H, int64_t W, int loop_form, int64_t* info);
+int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk,
+                            int64_t B, int64_t T, int64_t H, int64_t W, int loop_form, int rank_sort,
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Order-preserving integer ranks of q and k per column (b,h,w), the first stage of the f32
@@ -118,9 +133,9 @@ int l1attn_dense_column_ranks_f32(const float* q, const float* k, float* rq, flo
                                   int64_t B, int64_t T, int64_t H, int64_t W, void* stream);
 /*
  * The same ranks (identical rq, rk) from a merge sort written for this library instead of the library block
- * radix sort behind l1attn_dense_column_ranks_f32.  l1attn_dense_bwd_f32 uses it only when the environment
- * holds L1ATTN_RANK_SORT=merge (read once per process); kept beside the other until both have been timed on a
- * GPU.  No counterpart in the reference.
+ * radix sort behind l1attn_dense_column_ranks_f32.  l1attn_dense_bwd_f32 never uses it; l1attn_dense_bwd_ex_f32
+ * does with rank_sort = 1.  Kept beside the other until both have been timed on a GPU.  No counterpart in the
+ * reference.
  */
 int l1attn_dense_column_ranks_merge_f32(const float* q, const float* k, float* rq, float* rk,
                                         int64_t B, int64_t T, int64_t H, int64_t W, void* stream);

@@ -27,7 +27,9 @@ _ERR = {-1: "invalid argument", -2: "workspace missing or too small",
 #   rows16  float16 / bfloat16 rows in the sparse operators
 #   fused   l1attn_cuda.L1AttnFused (dense_fused_forward / dense_fused_backward)
 #   fixed   dense_forward_fixed (fixed-point float32 forward)
-EXPERIMENTAL = ("rows16", "fused", "fixed")
+#   bwd_pipe    set_dense_backward_form(loop_form=1 or 2): pipelined step loops of the long-sequence dense backward
+#   rank_merge  set_dense_backward_form(rank_sort=1): column ranks from the library's own merge sort
+EXPERIMENTAL = ("rows16", "fused", "fixed", "bwd_pipe", "rank_merge")
 _enabled = set(n for n in os.environ.get("L1ATTN_EXPERIMENTAL", "").replace(" ", "").split(",") if n)
 
 
@@ -77,6 +79,10 @@ def lib():
         L.l1attn_dense_bwd_workspace_bytes.argtypes = [_c_i64] * 4
         L.l1attn_dense_bwd_plan_info.restype = ctypes.c_int
         L.l1attn_dense_bwd_plan_info.argtypes = [_c_i64] * 4 + [_c_p]
+        L.l1attn_dense_bwd_plan_info_ex.restype = ctypes.c_int
+        L.l1attn_dense_bwd_plan_info_ex.argtypes = [_c_i64] * 4 + [ctypes.c_int, _c_p]
+        L.l1attn_dense_bwd_ex_f32.restype = ctypes.c_int
+        L.l1attn_dense_bwd_ex_f32.argtypes = [_c_p] * 5 + [_c_i64] * 4 + [ctypes.c_int] * 2 + [_c_p, _c_sz, _c_p]
         for sfx in ("f32", "f64"):
             f = getattr(L, "l1attn_dense_fwd_" + sfx)
             f.restype = ctypes.c_int
@@ -222,6 +228,33 @@ def dense_forward_fixed(q, k):
     return [attn]
 
 
+_dense_bwd_form = (0, 0)  # (loop_form, rank_sort) of l1attn_dense_bwd_ex_f32; (0, 0) is l1attn_dense_bwd_f32
+
+
+def set_dense_backward_form(loop_form=0, rank_sort=0):
+    """Which form of the float32 long-sequence backward dense_backward() runs from now on; returns the previous
+    (loop_form, rank_sort).  (0, 0) is the default entry point.  loop_form 1 / 2 (pipelined step loops) need
+    enable_experimental("bwd_pipe"), rank_sort 1 (merge sort for the column ranks) needs "rank_merge": those
+    kernels have not passed their GPU tests yet.  All forms give bit-identical gradients."""
+    global _dense_bwd_form
+    if loop_form not in (0, 1, 2) or rank_sort not in (0, 1):
+        raise ValueError("loop_form must be 0, 1 or 2 and rank_sort 0 or 1, got %r, %r" % (loop_form, rank_sort))
+    if loop_form:
+        _require_experimental("bwd_pipe", "the pipelined step loop of the dense backward")
+    if rank_sort:
+        _require_experimental("rank_merge", "the merge sort for the dense backward's column ranks")
+    old, _dense_bwd_form = _dense_bwd_form, (int(loop_form), int(rank_sort))
+    return old
+
+
+def dense_backward_plan(B, T, H, W, loop_form=None):
+    """l1attn_dense_bwd_plan_info_ex as a list of 16 ints, for the form dense_backward() currently runs."""
+    info = (ctypes.c_int64 * 16)()
+    form = _dense_bwd_form[0] if loop_form is None else int(loop_form)
+    check(lib().l1attn_dense_bwd_plan_info_ex(B, T, H, W, form, info), "l1attn_dense_bwd_plan_info_ex")
+    return list(info)
+
+
 def dense_backward(d_attn, q, k):
     """l1attn_cuda_drv.backward(d_attn, q, k) -> [d_q, d_k]  (cuda/l1attn_cuda_drv.cpp:67-104)."""
     check_input(d_attn, "d_attn")
@@ -239,9 +272,13 @@ def dense_backward(d_attn, q, k):
     with torch.cuda.device(q.device):
         ws_bytes = L.l1attn_dense_bwd_workspace_bytes(B, T, H, W) if sfx == "f32" else 0
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
-        rc = getattr(L, "l1attn_dense_bwd_" + sfx)(
-            ptr(d_attn), ptr(q), ptr(k), ptr(dq), ptr(dk), B, T, H, W,
-            ptr(ws) if ws is not None else None, ws_bytes, stream_of(q))
+        wsp = ptr(ws) if ws is not None else None
+        if sfx == "f32" and _dense_bwd_form != (0, 0):
+            rc = L.l1attn_dense_bwd_ex_f32(ptr(d_attn), ptr(q), ptr(k), ptr(dq), ptr(dk), B, T, H, W,
+                                           _dense_bwd_form[0], _dense_bwd_form[1], wsp, ws_bytes, stream_of(q))
+        else:
+            rc = getattr(L, "l1attn_dense_bwd_" + sfx)(
+                ptr(d_attn), ptr(q), ptr(k), ptr(dq), ptr(dk), B, T, H, W, wsp, ws_bytes, stream_of(q))
     check(rc, "l1attn_dense_bwd_" + sfx)
     return [dq, dk]
 

@@ -1034,32 +1034,10 @@ struct BwdPlan {
 
 constexpr int N_CU = 256;
 
-// Which kernel computes the column ranks of the long-sequence backward: the library block radix sort
-// (dense_rank.hip, the default: it is the one that has run the GPU tests) or the merge sort of rank_sort.hip
-// when the environment holds L1ATTN_RANK_SORT=merge.  Both give the same ranks; the choice is read once.
-bool l1_rank_sort_is_merge()
-{
-	static const bool merge = [] {
-		const char* e = getenv("L1ATTN_RANK_SORT");
-		return e && e[0] == 'm';
-	}();
-	return merge;
-}
-
-// Form of the branch-free step loop: one step of prefetch distance (the default: it is the one that has run the
-// GPU tests); two steps when the environment holds L1ATTN_BWD_PREFETCH=2; two steps, two LDS planes and one
-// barrier per step with L1ATTN_BWD_PREFETCH=3.  Same sums in the same order in all three, so the results are
-// bit-identical; the choice is read once.
-int l1_bwd_loop_form()
-{
-	static const int form = [] {
-		const char* e = getenv("L1ATTN_BWD_PREFETCH");
-		return (e && e[0] == '2') ? 1 : (e && e[0] == '3') ? 2 : 0;
-	}();
-	return form;
-}
-
-BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
+// loop_form: form of the branch-free step loop.  0: one step of prefetch distance (what l1attn_dense_bwd_f32
+// runs); 1: two steps; 2: two steps, two LDS planes and one barrier per step.  Same sums in the same order in all
+// three, so the results are bit-identical.  Shapes whose plan is not branch-free ignore it.
+BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W, int loop_form = 0)
 {
 	BwdPlan p{};
 	const int64_t HW = H * W;
@@ -1120,7 +1098,7 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W)
 	p.branch_free = p.wide && p.tt_rows == 64 && T % 64 == 0 && T % BWD_SJ == 0 && HW % p.threads == 0 &&
 	                (BWD_SJ * T + 128) * H < ((int64_t)1 << 29) &&
 	                p.threads % W == 0 && (int64_t)BWD_SJ * 64 * (p.threads / W) == (int64_t)4 * p.threads;
-	p.deep = (p.branch_free && T % (2 * BWD_SJ) == 0) ? l1_bwd_loop_form() : 0;
+	p.deep = (p.branch_free && T % (2 * BWD_SJ) == 0) ? loop_form : 0;
 	if (p.deep == 2) p.lds_bytes *= 2;
 	p.partial_bytes = p.n_tt > 1 ? (size_t)p.n_groups * T * HW * sizeof(float) : 0;
 	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
@@ -1295,12 +1273,12 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 	return p.per_batch_bytes * (size_t)nb;
 }
 
-int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64_t* info)
+int l1attn_dense_bwd_plan_info_ex(int64_t B, int64_t T, int64_t H, int64_t W, int loop_form, int64_t* info)
 {
-	if (!info || !shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	if (!info || !shape_ok(B, T, H, W) || loop_form < 0 || loop_form > 2) return L1ATTN_ERR_ARG;
 	for (int i = 0; i < 16; i++) info[i] = 0;
 	if (B * T * H * W == 0) return L1ATTN_OK;
-	const BwdPlan p = bwd_plan(B, T, H, W);
+	const BwdPlan p = bwd_plan(B, T, H, W, loop_form);
 	info[0] = p.fast;
 	if (!p.fast) return L1ATTN_OK;
 	info[1] = p.wide; info[2] = p.rank; info[3] = p.branch_free;
@@ -1312,15 +1290,23 @@ int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64
 	return L1ATTN_OK;
 }
 
-int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
-                         int64_t T, int64_t H, int64_t W, void* workspace, size_t workspace_bytes, void* stream)
+int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64_t* info)
 {
-	if (!shape_ok(B, T, H, W)) return L1ATTN_ERR_ARG;
+	return l1attn_dense_bwd_plan_info_ex(B, T, H, W, 0, info);
+}
+
+// rank_sort: 0 = column ranks from the library block radix sort (dense_rank.hip), 1 = from the merge sort of
+// rank_sort.hip; both give the same ranks
+int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
+                            int64_t T, int64_t H, int64_t W, int loop_form, int rank_sort, void* workspace,
+                            size_t workspace_bytes, void* stream)
+{
+	if (!shape_ok(B, T, H, W) || loop_form < 0 || loop_form > 2 || rank_sort < 0 || rank_sort > 1) return L1ATTN_ERR_ARG;
 	const int64_t n = B * T * H * W;
 	if (n == 0) return L1ATTN_OK;
 	if (!d_attn || !q || !k || !dq || !dk) return L1ATTN_ERR_ARG;
 	hipStream_t st = (hipStream_t)stream;
-	BwdPlan p = bwd_plan(B, T, H, W);
+	BwdPlan p = bwd_plan(B, T, H, W, loop_form);
 	if (!p.fast) return launch_bwd_generic<float>(d_attn, q, k, dq, dk, B, T, H, W, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
 	const int64_t HW = H * W;
@@ -1346,8 +1332,8 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 		const float* qa = q + b0 * T * HW;
 		const float* ka = k + b0 * T * HW;
 		if (p.rank) {
-			const int rc = l1_rank_sort_is_merge() ? l1_launch_column_ranks_merge(qa, ka, rq, rk, nb, T, H, W, st)
-			                                       : l1_launch_column_ranks(qa, ka, rq, rk, nb, T, H, W, st);
+			const int rc = rank_sort == 1 ? l1_launch_column_ranks_merge(qa, ka, rq, rk, nb, T, H, W, st)
+			                           : l1_launch_column_ranks(qa, ka, rq, rk, nb, T, H, W, st);
 			if (rc != L1ATTN_OK) return rc;
 			qa = rq;
 			ka = rk;
@@ -1380,6 +1366,12 @@ int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, fl
 		L1_LAUNCH_CHECK();
 	}
 	return L1ATTN_OK;
+}
+
+int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
+                         int64_t T, int64_t H, int64_t W, void* workspace, size_t workspace_bytes, void* stream)
+{
+	return l1attn_dense_bwd_ex_f32(d_attn, q, k, dq, dk, B, T, H, W, 0, 0, workspace, workspace_bytes, stream);
 }
 
 int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k, double* dq, double* dk, int64_t B,

@@ -406,7 +406,7 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
                           torch.zeros(B, E, H), 3, True)
     with pytest.raises(ValueError, match="unknown experimental"):
         drv.enable_experimental("everything")
-    assert drv.enable_experimental("rows16", "fused", "fixed") == frozenset(drv.EXPERIMENTAL)
+    assert drv.enable_experimental("rows16", "fused", "fixed") == frozenset(("rows16", "fused", "fixed"))
     a, = drv.dense_forward(q, k)
     assert a.shape == (B, T, T, H)
     a, = drv.dense_forward_fixed(q, k)
@@ -594,26 +594,55 @@ _Z4kernv: ; @k
         build.check_hot_loops(listing, (("kernv", 16, 2, 4.0),))
 
 
-def test_backward_variants_are_chosen_by_the_environment_only(lib):
-    """L1ATTN_BWD_PREFETCH=2 / =3 turn the branch-free plans into their pipelined forms (two steps of prefetch
-    distance; the same with two LDS planes, hence twice the LDS) and change nothing else; the variable is read
-    once per process, hence the child processes."""
-    code = ("import ctypes, sys; L = ctypes.CDLL(sys.argv[1]);"
-            "L.l1attn_dense_bwd_plan_info.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_void_p];"
-            "out = [];\n"
-            "for s in ((2, 64, 4, 32), (16, 1024, 8, 64), (8, 4096, 16, 64), (8, 4100, 16, 64), (2, 3, 16, 7)):\n"
-            "    a = (ctypes.c_int64 * 16)(); assert L.l1attn_dense_bwd_plan_info(*s, a) == 0; out.append(list(a))\n"
-            "print(out)")
-    import _l1attn_hip as drv
-    runs = {}
-    for value in ("", "2", "3", "7"):
-        env = dict(os.environ, L1ATTN_BWD_PREFETCH=value)
-        r = subprocess.run([sys.executable, "-c", code, drv._LIB_PATH], env=env, capture_output=True, text=True, check=True)
-        runs[value] = eval(r.stdout)
-    assert runs["7"] == runs[""] and all(p[14] == 0 for p in runs[""])          # unknown values mean the default
-    for form, value in ((1, "2"), (2, "3")):
-        for one, two in zip(runs[""], runs[value]):
+def test_backward_variants_are_chosen_by_argument_only(lib):
+    """loop_form 1 / 2 of l1attn_dense_bwd_plan_info_ex turn the branch-free plans into their pipelined forms (two
+    steps of prefetch distance; the same with two LDS planes, hence twice the LDS) and change nothing else.  The
+    library reads no environment variable: a process started with the old switches set plans as any other."""
+    shapes = ((2, 64, 4, 32), (16, 1024, 8, 64), (8, 4096, 16, 64), (8, 4100, 16, 64), (2, 3, 16, 7))
+    lib.l1attn_dense_bwd_plan_info.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_void_p]
+    lib.l1attn_dense_bwd_plan_info_ex.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_void_p]
+
+    def plans(form):
+        out = []
+        for s in shapes:
+            a = (ctypes.c_int64 * 16)()
+            rc = lib.l1attn_dense_bwd_plan_info(*s, a) if form is None else lib.l1attn_dense_bwd_plan_info_ex(*s, form, a)
+            assert rc == 0
+            out.append(list(a))
+        return out
+    runs = {f: plans(f) for f in (None, 0, 1, 2)}
+    assert runs[None] == runs[0] and all(p[14] == 0 for p in runs[0])
+    a = (ctypes.c_int64 * 16)()
+    assert lib.l1attn_dense_bwd_plan_info_ex(*shapes[1], 3, a) == -1 and lib.l1attn_dense_bwd_plan_info_ex(*shapes[1], -1, a) == -1
+    for form in (1, 2):
+        for one, two in zip(runs[0], runs[form]):
             assert two[14] == form * one[3]                                      # exactly the branch-free plans change
             assert two[11] == one[11] * (2 if two[14] == 2 else 1)               # LDS: two planes in form 2
             assert one[:11] + one[12:14] == two[:11] + two[12:14]                # and nothing else
-    assert [p[14] for p in runs["3"]] == [0, 2, 2, 0, 0]
+    assert [p[14] for p in runs[2]] == [0, 2, 2, 0, 0]
+    import _l1attn_hip as drv
+    code = ("import ctypes, sys; L = ctypes.CDLL(sys.argv[1]);"
+            "L.l1attn_dense_bwd_plan_info.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_void_p];"
+            "a = (ctypes.c_int64 * 16)(); assert L.l1attn_dense_bwd_plan_info(8, 4096, 16, 64, a) == 0; print(list(a))")
+    env = dict(os.environ, L1ATTN_BWD_PREFETCH="3", L1ATTN_RANK_SORT="merge")
+    r = subprocess.run([sys.executable, "-c", code, drv._LIB_PATH], env=env, capture_output=True, text=True, check=True)
+    assert eval(r.stdout) == runs[0][2]
+    with open(os.path.join(os.path.dirname(drv._LIB_PATH), "csrc", "dense.hip")) as f:
+        assert "getenv" not in f.read()
+
+
+def test_non_default_backward_forms_need_an_opt_in_by_name(monkeypatch):
+    import _l1attn_hip as drv
+    monkeypatch.setattr(drv, "_enabled", set())
+    monkeypatch.setattr(drv, "_dense_bwd_form", (0, 0))
+    with pytest.raises(RuntimeError, match="bwd_pipe"):
+        drv.set_dense_backward_form(loop_form=1)
+    with pytest.raises(RuntimeError, match="rank_merge"):
+        drv.set_dense_backward_form(rank_sort=1)
+    with pytest.raises(ValueError):
+        drv.set_dense_backward_form(loop_form=3)
+    assert drv.set_dense_backward_form(0, 0) == (0, 0)
+    drv.enable_experimental("bwd_pipe", "rank_merge")
+    assert drv.set_dense_backward_form(2, 1) == (0, 0) and drv._dense_bwd_form == (2, 1)
+    assert drv.dense_backward_plan(8, 4096, 16, 64)[14] == 2 and drv.dense_backward_plan(8, 4096, 16, 64, 0)[14] == 0
+    assert drv.set_dense_backward_form() == (2, 1)

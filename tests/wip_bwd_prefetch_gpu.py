@@ -7,10 +7,7 @@ This file has not run on a GPU yet, which is why its name keeps it out of pytest
 (run it as `python -m pytest tests/wip_bwd_prefetch_gpu.py -m gpu`); rename it to test_*.py once it has passed there.
 The kernels run on the CPU in tests/test_cpu_emulation_dense.py (AddressSanitizer and ThreadSanitizer).
 """
-import ctypes
 import os
-import subprocess
-import sys
 
 import pytest
 import torch
@@ -25,28 +22,28 @@ SHAPES = [((16, 1024, 8, 64), (0, 0)),     # second baseline configuration: sign
 
 
 @pytest.mark.parametrize("shape,kind", SHAPES)
-def test_two_step_prefetch_equals_the_default_backward(tmp_path, shape, kind):
-    """The prefetch distance is read from the environment once per process, so each run is a child process; both
-    write dq and dk of the same seeded problem, and the plan they ran on."""
-    code = (
-        "import sys, ctypes, torch; sys.path.insert(0, %r); import _l1attn_hip as drv;"
-        "B, T, H, W = %r; g = torch.Generator(device='cuda').manual_seed(5);"
-        "q = torch.randn(B, T, H, W, generator=g, device='cuda'); k = torch.randn(B, T, H, W, generator=g, device='cuda');"
-        "da = torch.empty(B, T, T, H, device='cuda');"
-        "[da[b].normal_(generator=g) for b in range(B)];"
-        "info = (ctypes.c_int64 * 16)(); assert drv.lib().l1attn_dense_bwd_plan_info(B, T, H, W, info) == 0;"
-        "dq, dk = drv.dense_backward(da, q, k); torch.cuda.synchronize();"
-        "torch.save([dq.cpu(), dk.cpu(), torch.tensor(list(info))], sys.argv[1])"
-        % (os.path.join(ROOT, "l1-attention_amd"), shape))
-    outs = []
-    for name, env in (("one_step", {}), ("two_steps", {"L1ATTN_BWD_PREFETCH": "2"}),
-                      ("two_steps_two_planes", {"L1ATTN_BWD_PREFETCH": "3"})):
-        path = str(tmp_path / (name + ".pt"))
-        print("case backward with prefetch distance:", name, shape, flush=True)
-        subprocess.run([sys.executable, "-c", code, path], check=True, env=dict(os.environ, **env), timeout=300)
-        outs.append(torch.load(path, weights_only=True))
-    (dq1, dk1, plan1), (dq2, dk2, plan2), (dq3, dk3, plan3) = outs
-    assert int(plan1[3]) == 1 and [int(p[14]) for p in (plan1, plan2, plan3)] == [0, 1, 2]   # branch-free; the three forms
-    assert (int(plan2[2]), int(int(plan2[9]) > 1)) == kind
-    assert torch.equal(dq1, dq2) and torch.equal(dk1, dk2)
-    assert torch.equal(dq1, dq3) and torch.equal(dk1, dk3)
+def test_two_step_prefetch_equals_the_default_backward(shape, kind):
+    """l1attn_dense_bwd_ex_f32 with loop_form 1 and 2 against the default entry point on the same seeded problem."""
+    import _l1attn_hip as drv
+    B, T, H, W = shape
+    plans = [drv.dense_backward_plan(B, T, H, W, f) for f in (0, 1, 2)]
+    assert plans[0][3] == 1 and [p[14] for p in plans] == [0, 1, 2]          # branch-free; the three forms
+    assert (plans[1][2], int(plans[1][9] > 1)) == kind
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k = (torch.randn(B, T, H, W, generator=g, device="cuda") for _ in range(2))
+    da = torch.empty(B, T, T, H, device="cuda")
+    for b in range(B):
+        da[b].normal_(generator=g)
+    print("case backward with prefetch distance: one_step", shape, flush=True)
+    dq1, dk1 = drv.dense_backward(da, q, k)
+    torch.cuda.synchronize()
+    drv.enable_experimental("bwd_pipe")
+    for form, name in ((1, "two_steps"), (2, "two_steps_two_planes")):
+        old = drv.set_dense_backward_form(loop_form=form)
+        try:
+            print("case backward with prefetch distance:", name, shape, flush=True)
+            dq2, dk2 = drv.dense_backward(da, q, k)
+            torch.cuda.synchronize()
+        finally:
+            drv.set_dense_backward_form(*old)
+        assert torch.equal(dq1, dq2) and torch.equal(dk1, dk2), name

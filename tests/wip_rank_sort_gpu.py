@@ -1,14 +1,12 @@
 """GPU parity of the merge-sort column-rank kernel (csrc/rank_sort.hip) against the library-sort kernel that the
-backward uses by default: the two must give identical rq and rk, and the whole backward with
-L1ATTN_RANK_SORT=merge must equal the default backward bit for bit.
+backward uses by default: the two must give identical rq and rk, and the whole backward through
+l1attn_dense_bwd_ex_f32(rank_sort=1) must equal the default backward bit for bit.
 
 This file has not run on a GPU yet, which is why its name keeps it out of pytest's collection
 (run it as `python -m pytest tests/wip_rank_sort_gpu.py -m gpu`); rename it to test_*.py once it has passed there.
 The kernel itself runs on the CPU in tests/test_cpu_emulation.py::test_merge_sort_column_ranks_on_cpu.
 """
 import os
-import subprocess
-import sys
 
 import pytest
 import torch
@@ -41,20 +39,24 @@ def test_merge_sort_ranks_equal_the_library_sort_ranks(shape):
     assert torch.equal(out[2], out[0]) and torch.equal(out[3], out[1])
 
 
-def test_backward_on_merge_sort_ranks_equals_the_default_backward(tmp_path):
-    """The choice of rank kernel is read from the environment once per process, so the merge-sort run is a child
-    process; both write dq and dk of the same seeded problem (rank path: T = 2048, 32 heads of 64 columns)."""
-    code = (
-        "import sys, torch; sys.path.insert(0, %r); import _l1attn_hip as drv;"
-        "g = torch.Generator().manual_seed(5); B, T, H, W = 3, 2048, 32, 64;"
-        "q = torch.randn(B, T, H, W, generator=g).cuda(); k = torch.randn(B, T, H, W, generator=g).cuda();"
-        "da = torch.randn(B, T, T, H, generator=g).cuda();"
-        "dq, dk = drv.dense_backward(da, q, k); torch.cuda.synchronize();"
-        "torch.save([dq.cpu(), dk.cpu()], sys.argv[1])" % os.path.join(ROOT, "l1-attention_amd"))
-    outs = []
-    for name, env in (("default", {}), ("merge", {"L1ATTN_RANK_SORT": "merge"})):
-        path = str(tmp_path / (name + ".pt"))
-        print("case backward with rank sort:", name, flush=True)
-        subprocess.run([sys.executable, "-c", code, path], check=True, env=dict(os.environ, **env), timeout=300)
-        outs.append(torch.load(path, weights_only=True))
-    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+def test_backward_on_merge_sort_ranks_equals_the_default_backward():
+    """l1attn_dense_bwd_ex_f32 with rank_sort = 1 against the default entry point on one seeded problem of the
+    rank path (T = 2048, 32 heads of 64 columns): bit-equal dq and dk."""
+    import _l1attn_hip as drv
+    B, T, H, W = 3, 2048, 32, 64
+    assert drv.dense_backward_plan(B, T, H, W)[2] == 1
+    g = torch.Generator().manual_seed(5)
+    q, k = (torch.randn(B, T, H, W, generator=g).cuda() for _ in range(2))
+    da = torch.randn(B, T, T, H, generator=g).cuda()
+    print("case backward with rank sort: default", flush=True)
+    dq0, dk0 = drv.dense_backward(da, q, k)
+    torch.cuda.synchronize()
+    drv.enable_experimental("rank_merge")
+    old = drv.set_dense_backward_form(rank_sort=1)
+    try:
+        print("case backward with rank sort: merge", flush=True)
+        dq1, dk1 = drv.dense_backward(da, q, k)
+        torch.cuda.synchronize()
+    finally:
+        drv.set_dense_backward_form(*old)
+    assert torch.equal(dq0, dq1) and torch.equal(dk0, dk1)
