@@ -81,45 +81,108 @@ def check_inline_asm_loads(asm_text, where=""):
     return with_sload
 
 
+def _kernel_bodies(asm_text):
+    """(kernel, [(line number, instruction text)], {label: index of the instruction it precedes}) for every
+    function of a device listing."""
+    cur, ins, labels = None, [], {}
+    for ln, line in enumerate(asm_text.split("\n"), 1):
+        l = line.strip()
+        if l.startswith("_Z") and ":" in l.split(";")[0]:
+            if cur is not None:
+                yield cur, ins, labels
+            cur, ins, labels = l.split(":")[0], [], {}
+            continue
+        if cur is None:
+            continue
+        if l.startswith(".Lfunc_end"):
+            yield cur, ins, labels
+            cur = None
+            continue
+        l = l.split(";")[0].strip()
+        m = re.match(r"^([.\w$]+):$", l)
+        if m:
+            labels[m.group(1)] = len(ins)
+        elif l and l[0] != ".":
+            ins.append((ln, l))
+    if cur is not None:
+        yield cur, ins, labels
+
+
+def _scalar_prefetch_step(l, inflight):
+    """One instruction against the SGPRs that still have a scalar load in flight before it:
+    (in-flight set after it, problem text or None, is a scalar load)."""
+    op = l.split()[0]
+    toks = re.findall(r"s\[\d+:\d+\]|s\d+", l)
+    used = set()
+    for t in toks:
+        used |= _sregs(t)
+    if op.startswith("s_load_dword") or op.startswith("s_buffer_load"):
+        # neither the address nor the destination may be in flight: two loads into one register complete in
+        # either order
+        bad = l if used & inflight else None
+        return inflight | (_sregs(toks[0]) if toks else set()), bad, True
+    if op == "s_waitcnt" and "lgkmcnt(0)" in l:
+        return frozenset(), None, False
+    if op == "s_endpgm":
+        return frozenset(), ("s_endpgm with scalar loads in flight" if inflight else None), False
+    if op in ("s_setpc_b64", "s_swappc_b64") and inflight:
+        return inflight, "indirect jump with scalar loads in flight: " + l, False
+    return inflight, (l if used & inflight else None), False
+
+
 def check_scalar_prefetch(asm_text, kernels=None):
     """Static check of the scalar loads in the generated ISA of the kernels that issue them from inline asm.
 
-    The pipelined forward kernels issue `s_load_dwordx16` from inline asm and wait for it one chunk of math later.
+    The pipelined kernels issue `s_load_dwordx16` from inline asm and wait for it one chunk of math later.
     The compiler does not know that the destination SGPRs are written asynchronously: if register
     pressure makes it spill, copy or reuse them between the load and the next `s_waitcnt lgkmcnt(0)`,
     the late-arriving data lands in whatever lives there by then (a pointer, an exec mask) and the
-    kernel faults.  This walks the kernels in `kernels` (a set of mangled names: build() passes every kernel
-    whose inline asm issues a scalar load, whatever its name or source file; None walks all, which only suits
-    straight-line listings since the walk does not follow branches) and fails the build if any instruction reads or
-    writes an SGPR that still has a scalar load in flight, or if the kernel ends with one in flight.
+    kernel faults.  This takes the kernels in `kernels` (a set of mangled names: build() passes every kernel
+    whose inline asm issues a scalar load, whatever its name or source file; None takes all) and follows their
+    control flow: the set of SGPRs with a load in flight is carried along the fall-through and along every
+    `s_branch` / `s_cbranch_*` edge, back edges included, joined by union where paths meet, until nothing
+    changes.  The build fails if on any path an instruction reads or writes an SGPR that is still in flight
+    (a second load into it included), or if the kernel can end with one in flight.
     Returns the number of scalar loads checked."""
-    cur, inflight, n_loads, problems = None, set(), 0, []
-    for kern, ln, l, _ in _walk_kernels(asm_text):
-        if kern != cur:
-            cur, inflight = kern, set()
-        if kernels is not None and cur not in kernels:
+    n_loads, problems = 0, []
+    for kern, ins, labels in _kernel_bodies(asm_text):
+        if (kernels is not None and kern not in kernels) or not ins:
             continue
-        op = l.split()[0]
-        toks = re.findall(r"s\[\d+:\d+\]|s\d+", l)
-        used = set()
-        for t in toks:
-            used |= _sregs(t)
-        if op.startswith("s_load_dword") or op.startswith("s_buffer_load"):
-            src = set()
-            for t in toks[1:]:
-                src |= _sregs(t)
-            if src & inflight:
-                problems.append((cur, ln, l))
-            inflight |= _sregs(toks[0]) if toks else set()
-            n_loads += 1
-        elif op == "s_waitcnt" and "lgkmcnt(0)" in l:
-            inflight = set()
-        elif op == "s_endpgm":
-            if inflight:
-                problems.append((cur, ln, "s_endpgm with scalar loads in flight"))
-            inflight = set()
-        elif used & inflight:
-            problems.append((cur, ln, l))
+        n = len(ins)
+
+        def successors(i):
+            op = ins[i][1].split()[0]
+            if op == "s_endpgm":
+                return []
+            m = re.match(r"s_c?branch\w*\s+([.\w$]+)", ins[i][1])
+            out = []
+            if m:
+                if m.group(1) not in labels:
+                    raise RuntimeError("scalar-prefetch check: %s line %d branches to an unknown label %s"
+                                       % (kern, ins[i][0], m.group(1)))
+                out.append(labels[m.group(1)])
+            if op != "s_branch" and i + 1 < n:
+                out.append(i + 1)
+            return out
+
+        state = [None] * n  # in-flight SGPRs before each instruction; None: not reached
+        state[0] = frozenset()
+        work = [0]
+        while work:
+            i = work.pop()
+            after = frozenset(_scalar_prefetch_step(ins[i][1], state[i])[0])
+            for s_ in successors(i):
+                joined = after if state[s_] is None else state[s_] | after
+                if joined != state[s_]:
+                    state[s_] = joined
+                    work.append(s_)
+        for i, (ln, l) in enumerate(ins):
+            if state[i] is None:
+                continue
+            _, bad, is_load = _scalar_prefetch_step(l, state[i])
+            n_loads += is_load
+            if bad:
+                problems.append((kern, ln, bad))
     if problems:
         msg = "\n".join("%s line %d: %s" % p for p in problems[:10])
         raise RuntimeError("scalar-prefetch check failed: SGPRs touched while their s_load is in flight\n" + msg)

@@ -216,6 +216,86 @@ _ZN1_18dense_fwd_f32_pipeILi64EEEv: ; @k
         build.check_scalar_prefetch(other.replace("	v_subrev_f32_e32 v1, s4, v2", "	s_mov_b32 s36, s2"))
 
 
+def test_scalar_prefetch_check_follows_branches_and_back_edges():
+    """The in-flight SGPR set is carried along every branch edge to a fixed point: violations that only exist on a
+    path through a loop's back edge, or in a block laid out after the exit, fail the build; a correct software
+    pipeline (load in the latch, wait at the loop header) passes."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "l1-attention_amd"))
+    import build
+    pipeline = """
+_Z4pipev: ; @k
+	s_load_dwordx2 s[0:1], s[4:5], 0x0
+	s_waitcnt lgkmcnt(0)
+	s_load_dwordx4 s[8:11], s[0:1], 0x0
+.LBB0_1:
+	HEADER
+	s_waitcnt lgkmcnt(0)
+	v_add_f32_e32 v1, s8, v1
+	s_mov_b32 s20, s9
+	s_add_u32 s0, s0, 16
+	s_load_dwordx4 s[8:11], s[0:1], 0x0
+	s_cmp_lt_u32 s0, s12
+	s_cbranch_scc1 .LBB0_1
+	s_waitcnt lgkmcnt(0)
+	s_endpgm
+.Lfunc_end0:
+"""
+    good = pipeline.replace("	HEADER\n", "	v_mov_b32_e32 v2, s20\n")
+    assert build.check_scalar_prefetch(good) == 3
+    # a copy at the loop header of a register the latch loads: clean on the way in, in flight on the back edge
+    for touch in ("s_mov_b32 s21, s8", "v_mov_b32_e32 v2, s11", "s_mov_b32 s10, 0"):
+        with pytest.raises(RuntimeError, match="in flight.*\n.*" + re.escape(touch)):
+            build.check_scalar_prefetch(pipeline.replace("HEADER", touch))
+    # a second load into registers whose first load has not been waited for
+    with pytest.raises(RuntimeError, match="in flight"):
+        build.check_scalar_prefetch(pipeline.replace("HEADER", "s_load_dword s9, s[0:1], 0x40"))
+    # the exit leaves the loop without its wait
+    with pytest.raises(RuntimeError, match="s_endpgm with scalar loads in flight"):
+        build.check_scalar_prefetch(good.replace("	s_waitcnt lgkmcnt(0)\n	s_endpgm", "	s_endpgm"))
+    # the latch laid out after the exit: the header is reached from it by s_branch only
+    rotated = """
+_Z3rotv: ; @k
+	s_load_dwordx2 s[0:1], s[4:5], 0x0
+	s_waitcnt lgkmcnt(0)
+	s_load_dwordx4 s[8:11], s[0:1], 0x0
+	s_waitcnt lgkmcnt(0)
+.LBB0_1:
+	HEADER
+	v_add_f32_e32 v1, s8, v1
+	s_cmp_lt_u32 s0, s12
+	s_cbranch_scc1 .LBB0_3
+	s_endpgm
+.LBB0_3:
+	s_add_u32 s0, s0, 16
+	s_load_dwordx4 s[8:11], s[0:1], 0x0
+	s_branch .LBB0_1
+.Lfunc_end0:
+"""
+    assert build.check_scalar_prefetch(rotated.replace("HEADER", "s_waitcnt lgkmcnt(0)")) == 3
+    with pytest.raises(RuntimeError, match="in flight.*\n.*line 9: v_add_f32_e32 v1, s8, v1"):
+        build.check_scalar_prefetch(rotated.replace("HEADER", "s_nop 0"))
+    # a wait on one arm of a branch does not cover the other arm
+    arms = """
+_Z4armsv: ; @k
+	s_load_dwordx2 s[2:3], s[4:5], 0x0
+	s_cbranch_scc1 .LBB0_2
+	s_waitcnt lgkmcnt(0)
+.LBB0_2:
+	s_mov_b32 s6, s2
+	s_waitcnt lgkmcnt(0)
+	s_endpgm
+.Lfunc_end0:
+"""
+    with pytest.raises(RuntimeError, match="s_mov_b32 s6, s2"):
+        build.check_scalar_prefetch(arms)
+    assert build.check_scalar_prefetch(arms.replace("	s_cbranch_scc1 .LBB0_2\n	s_waitcnt", "	s_waitcnt lgkmcnt(0)\n	s_cbranch_scc1 .LBB0_2\n	s_waitcnt")) == 1
+    with pytest.raises(RuntimeError, match="unknown label"):
+        build.check_scalar_prefetch(arms.replace(".LBB0_2:", ".LBB0_9:"))
+    # code no path reaches is not counted
+    assert build.check_scalar_prefetch(arms.replace("	s_cbranch_scc1 .LBB0_2\n", "	s_waitcnt lgkmcnt(0)\n	s_endpgm\n")) == 1
+
+
 def test_build_rejects_untracked_loads_in_inline_asm():
     """Loads whose result arrives later may not be issued from inline asm, in any kernel of any source: the
     compiler does not know the destination registers are still being written (a launch built that way took a GPU
