@@ -229,18 +229,64 @@ def check_asm_sources(files=None):
     return len(files)
 
 
-def isa_digests(asm_text):
+def kernarg_sgprs(asm_text):
+    """{kernel: first SGPR of the pair that holds the kernel-argument pointer at entry}, from the kernel
+    descriptors of a listing (user SGPRs are handed out in a fixed order: private segment buffer, dispatch
+    pointer, queue pointer, kernel-argument pointer)."""
+    out, cur, base = {}, None, 0
+    for raw in asm_text.split("\n"):
+        l = raw.strip()
+        if l.startswith(".amdhsa_kernel "):
+            cur, base = l.split()[1], 0
+        elif cur and l.startswith(".amdhsa_user_sgpr_"):
+            key, _, val = l.partition(" ")
+            width = {".amdhsa_user_sgpr_private_segment_buffer": 4, ".amdhsa_user_sgpr_dispatch_ptr": 2,
+                     ".amdhsa_user_sgpr_queue_ptr": 2}.get(key)
+            if width:
+                base += width * int(val)
+            elif key == ".amdhsa_user_sgpr_kernarg_segment_ptr" and int(val):
+                out[cur] = base
+        elif l.startswith(".end_amdhsa_kernel"):
+            cur = None
+    return out
+
+
+def isa_digests(asm_text, mask_kernarg_offsets=False):
     """{kernel: (sha256 of its instruction stream, number of instructions)} for a device listing: the instructions
     with their operands, in order, without comments, labels and directives.  Two builds whose digests agree run
-    the same machine code for that kernel."""
+    the same machine code for that kernel.  mask_kernarg_offsets: the immediate offset of every scalar load from
+    the kernel-argument pointer is left out of the digest, so that two kernels whose argument lists are laid out
+    differently and whose code is otherwise the same agree (runs of adjacent argument loads are compared in
+    sorted order)."""
     import hashlib
     streams = {}
+    karg = kernarg_sgprs(asm_text) if mask_kernarg_offsets else {}
+    overwritten = set()
     for kern, _, l, _ in _walk_kernels(asm_text):
         if re.match(r"^[\w.$]+:$", l):  # a label
             continue
         # branch targets carry the function's ordinal in the file (.LBB<ordinal>_<block>): drop the ordinal, so
         # that adding a kernel to a source does not change the digests of the others
-        streams.setdefault(kern, []).append(re.sub(r"\.LBB\d+_", ".LBB_", " ".join(l.split())))
+        l = re.sub(r"\.LBB\d+_", ".LBB_", " ".join(l.split()))
+        if kern in karg and kern not in overwritten:
+            l = re.sub(r"^(s_load_dword\w* \S+ s\[%d:%d\],) \S+" % (karg[kern], karg[kern] + 1), r"\1 KERNARG_OFFSET", l)
+            # the pair holds the argument pointer until the first instruction (in layout order) that names it as
+            # its destination; what is loaded through it afterwards is not a kernel argument
+            m = re.match(r"(?!s_cmp|s_bitcmp|s_cbranch|s_store)\S+ (s\[\d+:\d+\]|s\d+)\b", l)
+            if m and _sregs(m.group(1)) & {karg[kern], karg[kern] + 1}:
+                overwritten.add(kern)
+        streams.setdefault(kern, []).append(l)
+    if mask_kernarg_offsets:
+        # adjacent argument loads are independent of each other (each waits at its first use): their order in the
+        # listing follows the argument layout too, so a run of them is compared as a set
+        for v in streams.values():
+            i = 0
+            while i < len(v):
+                j = i
+                while j < len(v) and v[j].endswith(" KERNARG_OFFSET"):
+                    j += 1
+                v[i:j] = sorted(v[i:j])
+                i = j + 1
     return {k: (hashlib.sha256("\n".join(v).encode()).hexdigest()[:16], len(v)) for k, v in streams.items()}
 
 
@@ -431,8 +477,9 @@ def _build(verbose):
         # every kernel whose inline asm issues scalar loads no instruction touches an SGPR still in flight
         prefetchers = check_inline_asm_loads(text, os.path.basename(src))
         n += check_scalar_prefetch(text, prefetchers)
+        masked = isa_digests(text, mask_kernarg_offsets=True)
         for kname, (h, cnt) in sorted(isa_digests(text).items()):
-            digests.append("%s %s %s %d" % (os.path.basename(src), kname, h, cnt))
+            digests.append("%s %s %s %d %s" % (os.path.basename(src), kname, h, cnt, masked[kname][0]))
         if os.path.basename(src) == "dense.hip":
             asm = text
             if not any("dense_fwd_f32_pipe" in kname for kname in prefetchers):
@@ -449,7 +496,8 @@ def _build(verbose):
     with open(os.path.join(HERE, "build", "dense_kernel_resources.txt"), "w") as f:
         for name in sorted(res):
             f.write("%s %s\n" % (name, " ".join("%s=%d" % kv for kv in sorted(res[name].items()))))
-    # one line per kernel: source, mangled name, digest of its instruction stream, instruction count.  Kept under
+    # one line per kernel: source, mangled name, digest of its instruction stream, instruction count, the digest
+    # without the offsets of its kernel-argument loads.  Kept under
     # version control, so that the history shows which commits changed which kernel's machine code.
     with open(os.path.join(HERE, "isa_digests.txt"), "w") as f:
         f.write("\n".join(digests) + "\n")

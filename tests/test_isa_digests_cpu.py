@@ -20,8 +20,9 @@ NOW = os.path.join(ROOT, "l1-attention_amd", "isa_digests.txt")
 # Kernels of the tested set that exist in another form today.
 REPLACED = {
     # The pipelined forward gained a template flag and one kernel argument (the fixed-point variant's grid pointer):
-    # <W> is now <W, false>; its instruction stream differs from the tested one in the offsets of three
-    # kernel-argument loads and in nothing else (2079 instructions either way).
+    # <W> is now <W, false>; its instruction stream differs from the tested one in the offsets of the
+    # kernel-argument loads (and the order of two adjacent ones) and in nothing else: the digests that leave
+    # those offsets out are equal.
     "dense.hip dense_fwd_f32_pipe<32>": "dense.hip dense_fwd_f32_pipe<32, false>",
     "dense.hip dense_fwd_f32_pipe<64>": "dense.hip dense_fwd_f32_pipe<64, false>",
     "dense.hip dense_fwd_f32_pipe<96>": "dense.hip dense_fwd_f32_pipe<96, false>",
@@ -58,10 +59,11 @@ def test_gpu_tested_kernels_are_unchanged():
     if not os.path.exists(NOW) or shutil.which("c++filt") is None:
         pytest.skip("needs the digest table of a build and c++filt")
     gold = json.load(open(GOLD))
-    now = {}
+    now, now_masked = {}, {}
     for line in open(NOW):
-        src, mangled, digest, count = line.split()
+        src, mangled, digest, count, masked = line.split()
         now["%s %s" % (src, _short(mangled))] = (digest, int(count))
+        now_masked["%s %s" % (src, _short(mangled))] = (masked, int(count))
     assert len(gold["kernels"]) == 121 and len(now) >= 200
     same, moved = 0, []
     for name, (digest, count) in gold["kernels"].items():
@@ -70,10 +72,12 @@ def test_gpu_tested_kernels_are_unchanged():
             continue
         if name in REPLACED:
             d, c = now[REPLACED[name]]
-            assert c == count and d != digest  # same length; the argument offsets differ
+            assert c == count and d != digest  # same length; the argument offsets differ, and nothing else:
+            assert now_masked[REPLACED[name]] == tuple(gold["kernels_kernarg_offsets_masked"][name]), name
             moved.append(name)
             continue
         assert _today(name) in now, "kernel of the tested set is gone: " + name
         assert now[_today(name)] == (digest, count), "machine code changed since it ran on a GPU: " + name
+        assert now_masked[_today(name)] == tuple(gold["kernels_kernarg_offsets_masked"][name]), name
         same += 1
     assert same == 115 and len(moved) == 3
