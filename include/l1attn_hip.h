@@ -69,16 +69,21 @@ int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn,
  * each address of which is written by one lane only (where a workgroup adds several dst tiles into
  * one partial, the additions are done by the L2 in that lane's program order).  The partials are
  * held in `workspace` (device memory, 256-byte aligned, at least
- * l1attn_dense_bwd_workspace_bytes() for full speed; any multiple of one batch's share works,
- * the batches are then processed in several launches).  The f64 entry needs no workspace.
- * f32 tiled path (T >= 16 and H*W >= 32): sign() is taken as clamp(q*2^64 - k*2^64, -1, 1), exact for
- * |q|,|k| < 2^63 and differences that are 0 or at least 2^-64 in magnitude; a smaller non-zero
- * difference d enters with weight d*2^64 instead of +-1, larger magnitudes overflow (unspecified
- * result).  The generic f32 kernels (smaller shapes) and the f64 entry compare exactly.  For 2048 <= T <= 8192 (and enough work to fill
- * the GPU) sign() is taken from the column ranks of l1attn_dense_column_ranks_f32 instead, exact
- * for all finite inputs; the gradient is then assembled as 2*sum(hv*d_attn) - sum(d_attn) with
- * hv = (sign+1)/2, so an element whose pairs all tie comes out as a rounding residue of the two
- * sums (about 1e-6 of the largest gradient) instead of an exact zero.
+ * l1attn_dense_bwd_workspace_bytes() for full speed; its fixed head, info[15] of
+ * l1attn_dense_bwd_plan_info, plus any multiple of one batch's share, info[12], works: the batches
+ * are then processed in several launches).  The f64 entry needs no workspace.
+ * sign(): the generic f32 kernels (T < 16 or H*W < 32) and the f64 entry compare, as the reference does
+ * (cpp/l1attn_drv.cpp:7-11).  The f32 tiled path takes it as clamp(q*2^64 - k*2^64, -1, 1), which equals
+ * sign(q-k) for every pair while all magnitudes are below 2^63 and all non-zero ones at least 2^-41;
+ * a pre-pass over q and k checks exactly that on the device (a flag in the head of the workspace), and
+ * when it does not hold -- tiny values, huge ones, infinities, NaN -- two more kernels of the same call
+ * recompute dq and dk with comparisons.  The call stays asynchronous and the result is the reference's
+ * for every input; only the speed differs (O(T) reads per output element in the recomputation).
+ * For 2048 <= T <= 8192 (and enough work to fill the GPU) sign() is taken from the column ranks of
+ * l1attn_dense_column_ranks_f32 instead, exact for all finite inputs (no pre-pass, no flag); the
+ * gradient is then assembled as 2*sum(hv*d_attn) - sum(d_attn) with hv = (sign+1)/2, so an element
+ * whose pairs all tie comes out as a rounding residue of the two sums (about 1e-6 of the largest
+ * gradient) instead of an exact zero.
  */
 size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t W);
 /*
@@ -93,7 +98,7 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
  *  12 workspace bytes per batch              13 batches per launch with the full workspace
  *  14 form of the branch-free step loop the plan runs: 0 (always, through l1attn_dense_bwd_plan_info), or the
  *     loop_form given to l1attn_dense_bwd_plan_info_ex where the plan is branch-free
- *  15 reserved (0)
+ *  15 bytes at the head of the workspace that hold the sign-domain flag (256, or 0 with column ranks)
  * Returns 0, or a negative argument error.
  */
 int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64_t* info);

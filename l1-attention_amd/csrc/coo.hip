@@ -19,6 +19,12 @@
 #include "common.h"
 #include "plan.h"
 
+// The lanes named in `lanes` pass this point together.  Nothing on the GPU, where a wave's lanes execute every
+// instruction in lockstep; a host build that runs lanes as threads defines it as a barrier among those lanes.
+#ifndef L1_WAVE_LOCKSTEP
+#define L1_WAVE_LOCKSTEP(lanes) ((void)0)
+#endif
+
 namespace {
 
 constexpr int RS_THREADS = 256;
@@ -201,6 +207,7 @@ __global__ __launch_bounds__(RS_THREADS) void radix_scatter(const int* __restric
 		if (valid) {
 			const int prev = wcount[wave][d];  // read by every lane of the digit before the leader updates it
 			rank[c] = prev + __popcll(m & lt_mask);
+			L1_WAVE_LOCKSTEP(m);
 			if ((m & lt_mask) == 0) wcount[wave][d] = prev + __popcll(m);
 		}
 	}

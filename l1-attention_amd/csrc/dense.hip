@@ -129,6 +129,62 @@ __global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict_
 }
 
 // ------------------------------------------------------------------------------------------
+// Guard of the tiled fp32 backward that takes sign(q - k) from the scaled difference (dense_bwd_f32_fast without
+// column ranks): clamp(q*2^64 - k*2^64, -1, 1) equals sign(q - k) for every pair when all magnitudes are below
+// 2^63 (no overflow) and every non-zero value is at least 2^-41 in magnitude (then all values, and so all their
+// differences, are whole multiples of 2^-64).  dense_bwd_sign_domain sets *flag when some value of q or k is
+// outside that (NaN and infinities included); the two kernels after it then recompute dq and dk with exact
+// comparisons, as the generic kernels do, and return at once when the flag is clear.  The flag lives in the
+// caller's workspace and must be zero before dense_bwd_sign_domain runs.
+// ------------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(64) void dense_bwd_clear_flag(int* __restrict__ flag)
+{
+	if (threadIdx.x == 0 && blockIdx.x == 0) *flag = 0;
+}
+
+__global__ __launch_bounds__(256) void dense_bwd_sign_domain(const float* __restrict__ q, const float* __restrict__ k,
+                                                               int64_t n, int* __restrict__ flag)
+{
+	__shared__ int any_outside;
+	if (threadIdx.x == 0) any_outside = 0;
+	__syncthreads();
+	bool outside = false;
+	for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+		const float a = fabsf(q[i]), b = fabsf(k[i]);
+		// !(a < 2^63) is also true for NaN
+		outside |= !(a < 0x1p63f) || !(b < 0x1p63f) || (a != 0.0f && a < 0x1p-41f) || (b != 0.0f && b < 0x1p-41f);
+	}
+	if (outside) atomicOr(&any_outside, 1);
+	__syncthreads();
+	if (threadIdx.x == 0 && any_outside) atomicOr(flag, 1);
+}
+
+// DK false: one thread per dq element, src tokens summed in ascending order; DK true: one thread per dk element,
+// dst tokens in ascending order.  The arithmetic of dense_bwd_generic_dq / _dk.
+template <bool DK>
+__global__ __launch_bounds__(256) void dense_bwd_exact_if_flagged(const float* __restrict__ dA, const float* __restrict__ q,
+                                                                    const float* __restrict__ k, float* __restrict__ out,
+                                                                    int64_t B, int64_t Tn, int64_t H, int64_t W, float scale,
+                                                                    const int* __restrict__ flag)
+{
+	if (*flag == 0) return;
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= B * Tn * H * W) return;
+	const int64_t w = idx % W, h = (idx / W) % H, own = (idx / (W * H)) % Tn, b = idx / (W * H * Tn);
+	const float mine = DK ? k[idx] : q[idx];
+	float acc = 0;
+	for (int64_t o = 0; o < Tn; o++) {
+		const float other = (DK ? q : k)[((b * Tn + o) * H + h) * W + w];
+		const float ws = sgn_exact(DK ? other - mine : mine - other) * scale;
+		const int64_t s = DK ? own : o, t = DK ? o : own;
+		const float g = dA[((b * Tn + s) * Tn + t) * H + h];
+		if (DK) acc -= ws * g; else acc += ws * g;
+	}
+	out[idx] = acc;
+}
+
+// ------------------------------------------------------------------------------------------
 // fp32 forward, fast path
 // ------------------------------------------------------------------------------------------
 
@@ -1030,9 +1086,11 @@ struct BwdPlan {
 	size_t partial_bytes;    // partial-dk scratch for one batch (0 when a single dst tile)
 	size_t rank_bytes;       // rq and rk of one batch (0 unless rank)
 	size_t per_batch_bytes;  // workspace share of one batch
+	size_t flag_bytes;       // head of the workspace that holds the sign-domain flag (0 with column ranks)
 };
 
 constexpr int N_CU = 256;
+constexpr size_t BWD_FLAG_BYTES = 256;  // keeps what follows the flag 256-byte aligned
 
 // loop_form: form of the branch-free step loop.  0: one step of prefetch distance (what l1attn_dense_bwd_f32
 // runs); 1: two steps; 2: two steps, two LDS planes and one barrier per step.  Same sums in the same order in all
@@ -1104,6 +1162,7 @@ BwdPlan bwd_plan(int64_t B, int64_t T, int64_t H, int64_t W, int loop_form = 0)
 	// rq, rk [T][HW]; column sums per dst tile [n_tt][T][H] and their total [T][H]
 	p.rank_bytes = p.rank ? ((size_t)2 * T * HW + (size_t)(p.n_tt + 1) * T * H) * sizeof(float) : 0;
 	p.per_batch_bytes = p.partial_bytes + p.rank_bytes;
+	p.flag_bytes = p.rank ? 0 : BWD_FLAG_BYTES;
 	return p;
 }
 
@@ -1266,11 +1325,12 @@ size_t l1attn_dense_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 {
 	if (!shape_ok(B, T, H, W) || B * T * H * W == 0) return 0;
 	BwdPlan p = bwd_plan(B, T, H, W);
-	if (!p.fast || p.per_batch_bytes == 0) return 0;
+	if (!p.fast) return 0;
+	if (p.per_batch_bytes == 0) return p.flag_bytes;
 	// enough batches per launch to put >= 1024 workgroups in flight, never more than B
 	int64_t nb = l1_cdiv(1024, (int64_t)p.n_groups * p.n_cc);
 	if (nb > B) nb = B;
-	return p.per_batch_bytes * (size_t)nb;
+	return p.flag_bytes + p.per_batch_bytes * (size_t)nb;
 }
 
 int l1attn_dense_bwd_plan_info_ex(int64_t B, int64_t T, int64_t H, int64_t W, int loop_form, int64_t* info)
@@ -1287,6 +1347,7 @@ int l1attn_dense_bwd_plan_info_ex(int64_t B, int64_t T, int64_t H, int64_t W, in
 	info[12] = (int64_t)p.per_batch_bytes;
 	info[13] = p.per_batch_bytes ? std::min<int64_t>(B, l1_cdiv(1024, (int64_t)p.n_groups * p.n_cc)) : B;
 	info[14] = p.deep;
+	info[15] = (int64_t)p.flag_bytes;
 	return L1ATTN_OK;
 }
 
@@ -1310,13 +1371,38 @@ int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k,
 	if (!p.fast) return launch_bwd_generic<float>(d_attn, q, k, dq, dk, B, T, H, W, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
 	const int64_t HW = H * W;
+	const size_t need = p.flag_bytes + p.per_batch_bytes;
+	if (need && (!workspace || workspace_bytes < need)) return L1ATTN_ERR_WORKSPACE;
+	// Without column ranks the sign comes from the scaled difference: find out (on the device, without waiting)
+	// whether q and k are inside the range where that is exact; the fix-up launches at the end redo dq and dk
+	// with comparisons when they are not.
+	int* const flag = p.flag_bytes ? (int*)workspace : nullptr;
+	if (flag) {
+		hipLaunchKernelGGL(dense_bwd_clear_flag, dim3(1), dim3(64), 0, st, flag);
+		L1_LAUNCH_CHECK();
+		const dim3 dgrid((unsigned)std::min<int64_t>(l1_cdiv(n, 256 * 8), 4096));
+		hipLaunchKernelGGL(dense_bwd_sign_domain, dgrid, dim3(256), 0, st, q, k, n, flag);
+		L1_LAUNCH_CHECK();
+		workspace = (char*)workspace + p.flag_bytes;
+		workspace_bytes -= p.flag_bytes;
+	}
+	const auto fix_up = [&]() -> int {
+		if (!flag) return L1ATTN_OK;
+		const dim3 egrid((unsigned)l1_cdiv(n, 256));
+		hipLaunchKernelGGL(dense_bwd_exact_if_flagged<false>, egrid, dim3(256), 0, st, d_attn, q, k, dq, B, T, H, W, scale,
+		                   (const int*)flag);
+		L1_LAUNCH_CHECK();
+		hipLaunchKernelGGL(dense_bwd_exact_if_flagged<true>, egrid, dim3(256), 0, st, d_attn, q, k, dk, B, T, H, W, scale,
+		                   (const int*)flag);
+		L1_LAUNCH_CHECK();
+		return L1ATTN_OK;
+	};
 	if (p.per_batch_bytes == 0) {
 		dim3 grid(1, p.n_cc, (unsigned)B);
 		launch_bwd_fast(p, grid, st, d_attn, q, k, dq, dk, nullptr, (int)T, (int)H, (int)W, scale);
 		L1_LAUNCH_CHECK();
-		return L1ATTN_OK;
+		return fix_up();
 	}
-	if (!workspace || workspace_bytes < p.per_batch_bytes) return L1ATTN_ERR_WORKSPACE;
 	int64_t nb_max = (int64_t)(workspace_bytes / p.per_batch_bytes);
 	if (nb_max > B) nb_max = B;
 	// workspace: [n_groups][nb_max][T][HW] dk partials, then (rank path) rq and rk [nb_max][T][HW] each, the
@@ -1365,7 +1451,7 @@ int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k,
 #undef L1_REDUCE_CASE3
 		L1_LAUNCH_CHECK();
 	}
-	return L1ATTN_OK;
+	return fix_up();
 }
 
 int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,

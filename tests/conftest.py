@@ -32,7 +32,8 @@ CLANG = "/opt/rocm/llvm/bin/clang++"
 RUNNERS = {"fused": ("fused", "g++", "address,undefined"), "sparse": ("sparse", CLANG, "address,undefined"),
            "ranks": ("ranks", "g++", "address,undefined"), "dense": ("dense", "g++", "address,undefined"),
            "fused_tsan": ("fused", "g++", "thread"), "sparse_tsan": ("sparse", CLANG, "thread"),
-           "dense_tsan": ("dense", "g++", "thread"), "ranks_tsan": ("ranks", "g++", "thread")}
+           "dense_tsan": ("dense", "g++", "thread"), "ranks_tsan": ("ranks", "g++", "thread"),
+           "coo": ("coo", "g++", "address,undefined"), "coo_tsan": ("coo", "g++", "thread")}
 
 
 @pytest.fixture(scope="session")
@@ -101,3 +102,13 @@ def emu_dense_tsan(_emu_builds):
 @pytest.fixture(scope="session")
 def emu_ranks_tsan(_emu_builds):
     return _emu_runner(_emu_builds, "ranks_tsan")
+
+
+@pytest.fixture(scope="session")
+def emu_coo(_emu_builds):
+    return _emu_runner(_emu_builds, "coo")
+
+
+@pytest.fixture(scope="session")
+def emu_coo_tsan(_emu_builds):
+    return _emu_runner(_emu_builds, "coo_tsan")

@@ -5,16 +5,18 @@
 // __syncthreads() is a barrier among them, __shared__ arrays are static storage (workgroups run one
 // after the other).  It checks a kernel's index arithmetic, clamps, store predicates, LDS indexing,
 // barrier placement and launch geometry against exactly-sized host buffers; it says nothing about
-// timing, the memory model or the hardware.  Lanes of a wave do not run in lockstep here: a kernel
-// whose lanes hand values to each other through memory without a fence or a cross-lane operation in
-// between (the radix sort of coo.hip does, through per-wave LDS counters) cannot be run this way.  Never part of the library: only
-// tests/test_cpu_emulation.py builds with it.
+// timing, the memory model or the hardware.  Lanes of a wave do not run in lockstep here: where a kernel's
+// lanes hand values to each other through memory between two cross-lane operations (the radix sort of coo.hip
+// does, through per-wave LDS counters), the kernel marks the point with L1_WAVE_LOCKSTEP(lanes) -- nothing on the
+// GPU, a barrier among the named lanes here.  Never part of the library: only the tests build with it.
 #pragma once
 #include <math.h>
 #include <stddef.h>
 #include <stdio.h>
 #include <stdint.h>
+#include <string.h>
 #include <algorithm>
+#include <atomic>
 #include <barrier>
 #include <memory>
 #include <thread>
@@ -44,11 +46,21 @@ static inline float4 make_float4(float x, float y, float z, float w) { return fl
 struct double2 { double x, y; };
 static inline double2 make_double2(double x, double y) { return double2{x, y}; }
 struct uint2 { unsigned x, y; };
+struct int4 { int x, y, z, w; };
+static inline int4 make_int4(int x, int y, int z, int w) { return int4{x, y, z, w}; }
 
 typedef void* hipStream_t;
 typedef int hipError_t;
 #define hipSuccess 0
 static inline hipError_t hipGetLastError() { return hipSuccess; }
+// "device" memory is host memory and every launch has finished when it returns
+enum hipMemcpyKind { hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
+static inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t)
+{
+	memcpy(dst, src, n);
+	return hipSuccess;
+}
+static inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 
 namespace emu {
 inline thread_local dim3 threadIdx_;
@@ -66,7 +78,27 @@ inline bool dry = false;
 inline unsigned char* dynamic_lds = nullptr;  // the launch's dynamically sized LDS array, exactly `lds` bytes
 inline unsigned flat_tid() { return threadIdx_.x + blockDim_.x * (threadIdx_.y + blockDim_.y * threadIdx_.z); }
 inline void wave_sync() { wave_barrier[flat_tid() >> 6]->arrive_and_wait(); }
+// Barrier among a subset of a wave's lanes, keyed by the subset's lowest lane (disjoint subsets of one wave may
+// wait at the same time): the last lane to arrive opens the gate for the others.
+struct LaneGate { std::atomic<int> count{0}, generation{0}; };
+inline std::unique_ptr<LaneGate[]> lane_gates;  // 64 per wave
+inline void lockstep(unsigned long long lanes)
+{
+	const unsigned tid = flat_tid(), lane = tid & 63u;
+	if (!((lanes >> lane) & 1ull)) abort();  // the caller must be one of the lanes it names
+	const int n = __builtin_popcountll(lanes);
+	LaneGate& g = lane_gates[(tid & ~63u) + (unsigned)__builtin_ctzll(lanes)];
+	const int gen = g.generation.load();
+	if (g.count.fetch_add(1) + 1 == n) {
+		g.count.store(0);
+		g.generation.fetch_add(1);
+		g.generation.notify_all();
+	} else {
+		while (g.generation.load() == gen) g.generation.wait(gen);
+	}
 }
+}
+#define L1_WAVE_LOCKSTEP(lanes) emu::lockstep(lanes)
 #define threadIdx (emu::threadIdx_)
 #define blockIdx (emu::blockIdx_)
 #define blockDim (emu::blockDim_)
@@ -94,6 +126,47 @@ static inline T __shfl_xor(T x, int lane_mask)
 	const T r = (T)emu::wave_slots[base + ((tid ^ (unsigned)lane_mask) & 63u)];
 	emu::wave_sync();
 	return r;
+}
+template <typename T>
+static inline T __shfl_xor(T x, int lane_mask, int width)
+{
+	if (width != 64) abort();
+	return __shfl_xor(x, lane_mask);
+}
+// value of the lane `delta` below, or the lane's own where there is none.  Every lane of the wave must call it.
+template <typename T>
+static inline T __shfl_up(T x, unsigned delta, int width)
+{
+	if (width != 64) abort();
+	const unsigned tid = emu::flat_tid();
+	emu::wave_slots[tid] = (double)x;
+	emu::wave_sync();
+	const T r = (tid & 63u) >= delta ? (T)emu::wave_slots[tid - delta] : x;
+	emu::wave_sync();
+	return r;
+}
+// bit l = predicate of lane l.  Every lane of the wave must call it (the emulated waves are always full or end
+// with the workgroup: a lane beyond it reads as 0).
+static inline unsigned long long __ballot(int pred)
+{
+	const unsigned tid = emu::flat_tid(), base = tid & ~63u;
+	emu::wave_slots[tid] = pred ? 1.0 : 0.0;
+	emu::wave_sync();
+	unsigned long long m = 0;
+	for (unsigned l = 0; l < 64 && base + l < emu::wave_slots.size(); l++)
+		if (emu::wave_slots[base + l] != 0.0) m |= 1ull << l;
+	emu::wave_sync();
+	return m;
+}
+static inline int __popcll(unsigned long long x) { return __builtin_popcountll(x); }
+// atomics on global and LDS words: the return value is the old one
+static inline int atomicAdd(int* p, int v) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); }
+static inline int atomicOr(int* p, int v) { return __atomic_fetch_or(p, v, __ATOMIC_SEQ_CST); }
+static inline int atomicMax(int* p, int v)
+{
+	int old = __atomic_load_n(p, __ATOMIC_SEQ_CST);
+	while (old < v && !__atomic_compare_exchange_n(p, &old, v, false, __ATOMIC_SEQ_CST, __ATOMIC_SEQ_CST)) {}
+	return old;
 }
 // DPP row shift right by n (control 0x110 + n) with out-of-row lanes reading zero: lane l of each aligned group
 // of sixteen receives the value of lane l - n of the same group.  Every lane of the wave must call it.
@@ -170,6 +243,7 @@ static inline void emu_launch(const char* name, K kernel, dim3 grid, dim3 block,
 				for (unsigned w = 0; w < (nt + 63) / 64; w++)
 					emu::wave_barrier.emplace_back(new std::barrier<>(std::min(64u, nt - w * 64)));
 				emu::wave_slots.assign((nt + 63) / 64 * 64, 0.0);
+				emu::lane_gates.reset(new emu::LaneGate[(nt + 63) / 64 * 64]);
 			}
 			step.arrive_and_wait();
 			kernel(args...);

@@ -1,7 +1,7 @@
 // TEST INFRASTRUCTURE: host stand-ins for the entry points of csrc/coo.hip and csrc/version.hip in the emulated
-// library.  The radix sort of coo.hip hands values between the lanes of a wave through LDS in lockstep, which OS
-// threads cannot stand for; these functions produce what those kernels are specified to produce (the plan layout
-// of csrc/plan.h, expandCoo's ranks) with plain loops.  They check nothing about coo.hip.
+// library.  These functions produce what those kernels are specified to produce (the plan layout of csrc/plan.h,
+// expandCoo's ranks) with plain loops, which keeps whole-operator runs on the emulated library short.  They check
+// nothing about coo.hip: its kernels run from source in tests/test_cpu_emulation_coo.py (run_coo.cpp).
 #include "hip/hip_runtime.h"
 #include "../../l1-attention_amd/csrc/plan.h"
 #include <map>

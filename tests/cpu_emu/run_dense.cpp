@@ -6,7 +6,8 @@
 //                                       backward and fixed-point forward would make is checked against the limits
 //                                       of a HIP launch and printed (kernel, grid, block, LDS bytes); nothing runs
 // in : int64 B,T,H,W then q,k [B,T,H,W] and dA [B,T,T,H] in the chosen type (fixed: float32)
-// out: attn [B,T,T,H], dq, dk [B,T,H,W] (fixed: attn only), then int64[16] of l1attn_dense_bwd_plan_info
+// out: attn [B,T,T,H], dq, dk [B,T,H,W] (fixed: attn only), then int64[16] of l1attn_dense_bwd_plan_info and one
+//      int64: the sign-domain flag the backward left in its workspace (-1 where the plan keeps none)
 // Every buffer is malloc'ed at its exact size and every output starts as NaN, so AddressSanitizer reports an
 // access outside a buffer and the caller sees an element that was never written.
 //
@@ -165,6 +166,7 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, const char* mode, int argc,
 	if (fread(q, sizeof(F), n, fi) != n || fread(k, sizeof(F), n, fi) != n || fread(dA, sizeof(F), na, fi) != na) return 3;
 	F *attn = alloc_nan<F>(na), *dq = alloc_nan<F>(n), *dk = alloc_nan<F>(n);
 	int rc = 0;
+	int64_t domain_flag = -1;  // the backward's sign-domain flag after the call; -1: the plan keeps none
 	if constexpr (sizeof(F) == 8) {
 		rc = l1attn_dense_fwd_f64(q, k, attn, B, T, H, W, nullptr);
 		if (!rc) rc = l1attn_dense_bwd_f64(dA, q, k, dq, dk, B, T, H, W, nullptr, 0, nullptr);
@@ -186,7 +188,11 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, const char* mode, int argc,
 		} else if (!rc) {
 			const size_t wb = l1attn_dense_bwd_workspace_bytes(B, T, H, W);
 			void* wsb = wb ? aligned_alloc(256, (wb + 255) / 256 * 256) : nullptr;
+			if (wsb) memset(wsb, 0xA5, wb);  // nothing may rest on a zeroed workspace
 			rc = l1attn_dense_bwd_f32(dA, q, k, dq, dk, B, T, H, W, wsb, wb, nullptr);
+			int64_t info[16];
+			l1attn_dense_bwd_plan_info(B, T, H, W, info);
+			if (!rc && info[15] > 0) domain_flag = *(const int*)wsb;
 			free(wsb);
 		}
 	}
@@ -200,6 +206,7 @@ static int run(FILE* fi, FILE* fo, const int64_t* d, const char* mode, int argc,
 	int64_t info[16];
 	l1attn_dense_bwd_plan_info(B, T, H, W, info);
 	fwrite(info, sizeof(int64_t), 16, fo);
+	fwrite(&domain_flag, sizeof(int64_t), 1, fo);
 	free(q); free(k); free(dA); free(attn); free(dq); free(dk);
 	return 0;
 }

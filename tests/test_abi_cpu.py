@@ -50,10 +50,12 @@ def test_host_side_argument_logic(lib):
     assert lib.l1attn_version() >= 100
     lib.l1attn_dense_bwd_workspace_bytes.restype = sz
     lib.l1attn_dense_bwd_workspace_bytes.argtypes = [i64] * 4
-    # one dst tile (T <= 32) or the generic path needs no workspace
-    assert lib.l1attn_dense_bwd_workspace_bytes(2, 32, 4, 32) == 0
+    # one dst tile (T <= 32) needs the 256 bytes of the sign-domain flag only, the generic path no workspace
+    assert lib.l1attn_dense_bwd_workspace_bytes(2, 32, 4, 32) == 256
     assert lib.l1attn_dense_bwd_workspace_bytes(2, 3, 16, 7) == 0
-    # headline config: 64 dst tiles (64 tokens each) x 8 batches x T x H*W floats
+    # second baseline configuration (no column ranks): the flag, then 16 dk partials [T][HW] for each of the 16 batches
+    assert lib.l1attn_dense_bwd_workspace_bytes(16, 1024, 8, 64) == 256 + 16 * 16 * 1024 * 512 * 4
+    # headline config (column ranks, no flag): 64 dst tiles (64 tokens each) x 8 batches x T x H*W floats
     # per batch: 16 dk partials [T][HW] (64 dst tiles, four per workgroup), the two rank arrays [T][HW],
     # 64 + 1 column-sum arrays [T][H]
     assert lib.l1attn_dense_bwd_workspace_bytes(8, 4096, 16, 64) == 8 * 4 * ((16 + 2) * 4096 * 1024 + 65 * 4096 * 16)
@@ -79,7 +81,7 @@ def _plan(lib, B, T, H, W):
     a = (ctypes.c_int64 * 16)()
     assert lib.l1attn_dense_bwd_plan_info(B, T, H, W, a) == 0
     keys = ("tiled", "wide", "rank", "branch_free", "threads", "n_cc", "n_tt", "tt_rows", "per", "group", "n_groups",
-            "lds_bytes", "per_batch_bytes", "batches_per_launch", "deep")
+            "lds_bytes", "per_batch_bytes", "batches_per_launch", "deep", "flag_bytes")
     return dict(zip(keys, list(a)))
 
 
@@ -142,7 +144,8 @@ def test_dense_backward_plan_invariants_over_a_shape_grid(lib):
                     assert p["per_batch_bytes"] == partial + ranks
                     nb = min(B, cdiv(1024, p["n_groups"] * p["n_cc"])) if p["per_batch_bytes"] else B
                     assert p["batches_per_launch"] == nb
-                    assert lib.l1attn_dense_bwd_workspace_bytes(B, T, H, W) == p["per_batch_bytes"] * nb
+                    assert p["flag_bytes"] == (0 if p["rank"] else 256)       # the scaled-difference sign keeps a flag
+                    assert lib.l1attn_dense_bwd_workspace_bytes(B, T, H, W) == p["flag_bytes"] + p["per_batch_bytes"] * nb
     # the grid reaches every family of instantiations: narrow, wide, ranks, branch-free, grouped
     assert (0, 0, 0, False) in seen and (1, 0, 0, False) in seen and (1, 1, 0, False) in seen
     assert (1, 1, 1, True) in seen and (1, 0, 1, True) in seen and (1, 1, 1, False) in seen and (1, 0, 1, False) in seen

@@ -57,7 +57,8 @@ def _run(exe, d, shape, mode="f32", extra=(), seed=0, ties=False, scale=1.0, inp
         out["dq"] = torch.from_numpy(np.frombuffer(raw, npdt, n, off).reshape(B, T, H, W).copy())
         out["dk"] = torch.from_numpy(np.frombuffer(raw, npdt, n, off + n * it).reshape(B, T, H, W).copy())
         off += 2 * n * it
-    assert len(raw) == off + 16 * 8
+    assert len(raw) == off + 17 * 8
+    out["domain_flag"] = int(np.frombuffer(raw, np.int64, 1, off + 16 * 8)[0])
     keys = ("tiled", "wide", "rank", "branch_free", "threads", "n_cc", "n_tt", "tt_rows", "per", "group", "n_groups")
     out["plan"] = dict(zip(keys, np.frombuffer(raw, np.int64, 16, off).tolist()))
     return out
@@ -119,6 +120,41 @@ def test_dense_float64_and_ties(runner, tmp_path):
     assert float((r["q"][:, :, None] == r["k"][:, None]).float().mean()) > 0.1  # sign(0) = 0 matters here
     _check(r, 1e-6, 1e-5)
     _check(_run(runner, tmp_path, (1, 33, 2, 7), ties=True, seed=9), 1e-6, 1e-5)  # untiled kernels, exact compares
+
+
+def test_sign_domain_guard_of_the_tiled_backward(runner, tmp_path):
+    """The tiled float32 backward without column ranks takes sign(q - k) from the difference of q * 2^64 and
+    k * 2^64, which is exact while every magnitude is below 2^63 and every non-zero one at least 2^-41.  A pre-pass
+    raises a flag in the workspace otherwise and two fix-up kernels redo dq and dk with comparisons, so the result is
+    the reference's sign() (cpp/l1attn_drv.cpp:7-11) for every input: tiny values whose differences the scaling
+    would leave fractional, magnitudes it would overflow, infinities.  Inside the range the flag stays clear and
+    the fix-up kernels leave the tiled result alone."""
+    shape = (2, 64, 4, 32)                                                    # 32-token tiles, two per sequence
+    g = torch.Generator().manual_seed(31)
+    q0, k0 = (torch.randn(*shape, generator=g) for _ in range(2))
+    k0[0, 1] = q0[0, 2]                                                       # exact ties stay exact under powers of two
+    dA = torch.randn(2, 64, 64, 4, generator=g)
+    for e, flagged in ((0, 0), (-20, 0), (40, 0), (-36, 1), (-70, 1), (64, 1)):   # (2^-36: some values below 2^-41)
+        r = _run(runner, tmp_path, shape, inputs=(q0 * 2.0 ** e, k0 * 2.0 ** e, dA))
+        assert r["plan"]["tiled"] == 1 and r["plan"]["rank"] == 0 and r["domain_flag"] == flagged, e
+        rdq, rdk = oracle.dense_bwd(dA.double(), r["q"].double(), r["k"].double())
+        assert cf.rel_err(r["dq"], rdq) <= 1e-4 and cf.rel_err(r["dk"], rdk) <= 1e-4, e
+    # one value outside the range is enough: a subnormal, a value of 2^63, an infinity in k
+    for where, value in (((1, 63, 3, 31), 1e-40), ((0, 0, 0, 0), 2.0 ** 63), ((1, 5, 2, 7), float("inf"))):
+        q, k = q0.clone(), k0.clone()
+        (q if value != float("inf") else k)[where] = value
+        r = _run(runner, tmp_path, shape, inputs=(q, k, dA))
+        assert r["domain_flag"] == 1
+        rdq, rdk = oracle.dense_bwd(dA.double(), q.double(), k.double())
+        assert cf.rel_err(r["dq"], rdq) <= 1e-4 and cf.rel_err(r["dk"], rdk) <= 1e-4, value
+    # exact zeros are inside the range (|0 - x| is a whole multiple of 2^-64 whenever x is)
+    q = q0.clone()
+    q[:, ::3] = 0.0
+    assert _run(runner, tmp_path, shape, inputs=(q, k0, dA))["domain_flag"] == 0
+    # plans that keep no flag: the untiled kernels compare exactly whatever the range
+    r = _run(runner, tmp_path, (1, 12, 2, 7), scale=2.0 ** -70, seed=3)
+    assert r["plan"]["tiled"] == 0 and r["domain_flag"] == -1
+    _check(r, 1e-5, 1e-4)
 
 
 def test_dense_kernels_against_the_reference_extension_golden_vectors(runner, tmp_path):
@@ -248,6 +284,9 @@ def test_dense_kernels_under_thread_sanitizer(tmp_path, emu_dense_tsan):
     _check(_run(exe, d, (1, 256, 2, 64), extra=("wide", 64, 1, 4, "deep2"), seed=8), 1e-5, 1e-4)
     _check(_run(exe, d, (3, 128, 2, 64), extra=("wide", 64, 0, 2, "deep2"), seed=9), 1e-5, 1e-4)
     _check(_run(exe, d, (1, 64, 2, 64), mode="fixed", seed=5), 1e-5, None)
+    r = _run(exe, d, (1, 64, 4, 32), seed=1, scale=2.0 ** -70)   # sign-domain flag raised: the fix-up kernels run
+    assert r["domain_flag"] == 1
+    _check(r, 1e-5, 1e-4)
 
 
 def _dims(exe, shape):
@@ -271,8 +310,14 @@ def test_launch_geometry_at_full_size(runner):
                             ("dense_bwd_f32_fast<64, 512, 4, true, true, true>", (16, 2, 8), 512, 4 * 8 * 68 * 4),
                             ("dense_bwd_reduce_colsum", (2048, 1, 1), 256, 0),
                             ("dense_bwd_reduce_dk<true, true, false>", (32768, 1, 1), 256, 0)]
+    # without column ranks the backward brackets its kernels with the sign-domain check and the exact fix-up
     rcs, launches = _dims(runner, (16, 1024, 8, 64))
-    assert rcs["backward"] == "0" and launches[1] == ("dense_bwd_f32_fast<64, 512, 4, false, false, true>", (16, 1, 16), 512, 8704)
+    assert rcs["backward"] == "0" and [l[0] for l in launches[1:]][:7] == [
+        "dense_bwd_clear_flag", "dense_bwd_sign_domain", "dense_bwd_f32_fast<64, 512, 4, false, false, true>",
+        "dense_bwd_reduce_dk<true, false, false>", "dense_bwd_exact_if_flagged<false>", "dense_bwd_exact_if_flagged<true>",
+        "fixed_absmax"]
+    assert launches[3] == ("dense_bwd_f32_fast<64, 512, 4, false, false, true>", (16, 1, 16), 512, 8704)
+    assert launches[2][1] == (4096, 1, 1) and launches[5][1] == (16 * 1024 * 8 * 64 // 256, 1, 1)
     assert _dims(runner, (2, 64, 4, 32))[0]["backward"] == "0"
     kernels = set()
     for T in (16, 32, 64, 128, 256):

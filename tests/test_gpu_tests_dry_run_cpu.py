@@ -37,8 +37,11 @@ def test_sign_range_test_walks_on_a_model_of_the_kernel(gpu_tests_on_cpu, monkey
     def model(q, k, da):
         W = q.shape[-1]
         scale = -1 / math.sqrt(W)
-        if q.dtype == torch.float64 or q.shape[2] * W < 32:      # exact comparisons
+        x = torch.cat([q.flatten(), k.flatten()]).abs()
+        outside = bool((~(x < 2.0 ** 63)).any() or ((x != 0) & (x < 2.0 ** -41)).any())   # what the pre-pass flags
+        if q.dtype == torch.float64 or q.shape[2] * W < 32 or outside:                      # exact comparisons
             s = torch.sign(q[:, None].double() - k[:, :, None].double())
+            s = torch.nan_to_num(s, nan=0.0)                                                  # inf - inf: neither > 0 nor < 0
         else:                                                     # float32: clamp((q*2^64 - k*2^64), -1, 1)
             s = ((q * 2.0 ** 64)[:, None] - (k * 2.0 ** 64)[:, :, None]).clamp(-1, 1).double()
         dq = scale * torch.einsum("bsthw,bsth->bthw", s, da.double())

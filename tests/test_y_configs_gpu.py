@@ -73,43 +73,39 @@ def _dense_bwd_gpu(q, k, da):
 
 def test_sign_domain_of_the_fast_float32_backward():
     """The float32 backward below 2048 tokens takes sign(q-k) as clamp((q - k) * 2^64, -1, 1) with q and k scaled
-    first: exact for |q|, |k| < 2^63 and for differences that are 0 or at least 2^-64 in magnitude, which this test
-    shows at both ends of a wide range (inputs scaled by 2^-36 and 2^40 match the oracle, whose sign() is a
-    comparison: cpp/l1attn_drv.cpp:7-11).  Below the range the clamp does not saturate and the gradient follows the
-    stated formula instead of the sign (inputs scaled by 2^-70: checked against that formula, and shown to differ
-    from the oracle); above it the scaled values overflow and the result is unspecified.  The float64 entry point and
-    the generic float32 kernels (fewer than 16 tokens or fewer than 32 columns per token) compare exactly and have no
-    such range (checked at both scales)."""
+    first: exact while every magnitude is below 2^63 and every non-zero one at least 2^-41 (inputs scaled by 2^-20
+    and 2^40 are inside).  A pre-pass of the same call checks that on the device, and outside it -- inputs scaled by
+    2^-70, whose differences the scaling leaves fractional; by 2^64, which it overflows; one subnormal or infinite
+    value -- dq and dk are recomputed with comparisons, so every case matches the oracle, whose sign() is the
+    reference's comparison (cpp/l1attn_drv.cpp:7-11).  The float64 entry point and the generic float32 kernels
+    (fewer than 16 tokens or fewer than 32 columns per token) compare exactly to begin with."""
     print("case sign domain", flush=True)
     import _l1attn_hip as drv
     B, T, H, W = 1, 192, 8, 64
     info = (drv.ctypes.c_int64 * 16)()
     assert drv.lib().l1attn_dense_bwd_plan_info(B, T, H, W, info) == 0
-    assert info[0] == 1 and info[2] == 0          # tiled path without column ranks: the form described above
+    assert info[0] == 1 and info[2] == 0 and info[15] == 256   # tiled path without column ranks: the form described above
     g = torch.Generator().manual_seed(77)
     q0, k0 = torch.randn(B, T, H, W, generator=g), torch.randn(B, T, H, W, generator=g)
     k0[0, 1] = q0[0, 2]                            # exact ties stay exact under scaling by powers of two
     da = torch.randn(B, T, T, H, generator=g)
-    scale = -1.0 / math.sqrt(W)
-    d0 = (q0[:, None].double() - k0[:, :, None].double()).abs()
-    d0_min = float(d0[d0 > 0].min())              # 2^-22 for this seed
-    for e in (-36, 40):
-        assert d0_min * 2.0 ** (e + 64) >= 1.0 and float(q0.abs().max()) * 2.0 ** e < 2.0 ** 63   # inside the range
+    for e in (-20, 40, -70, 64):
+        print("case sign domain: inputs scaled by 2^%d" % e, flush=True)
         q, k = q0 * 2.0 ** e, k0 * 2.0 ** e
+        x = torch.cat([q.flatten(), k.flatten()]).abs()
+        inside = float(x.max()) < 2.0 ** 63 and float(x[x != 0].min()) >= 2.0 ** -41
+        assert inside == (e in (-20, 40))
         dq, dk = _dense_bwd_gpu(q, k, da)
         rdq, rdk = oracle.dense_bwd(da.double(), q.double(), k.double())
         assert cf.rel_err(dq, rdq) <= cc.BWD_TOL and cf.rel_err(dk, rdk) <= cc.BWD_TOL, e
-    # below the range: the documented formula, not the sign
-    q, k = q0 * 2.0 ** -70, k0 * 2.0 ** -70
-    dq, dk = _dense_bwd_gpu(q, k, da)
-    qs, ks = (q.double() * 2.0 ** 64).to(DEV), (k.double() * 2.0 ** 64).to(DEV)
-    s = (qs[:, None] - ks[:, :, None]).float().double().clamp(-1.0, 1.0)       # [B,S,T,H,W], rounded like the fp32 subtraction
-    fdq = scale * torch.einsum("bsthw,bsth->bthw", s, da.double().to(DEV)).cpu()
-    fdk = -scale * torch.einsum("bsthw,bsth->bshw", s, da.double().to(DEV)).cpu()
-    assert cf.rel_err(dq, fdq) <= cc.BWD_TOL and cf.rel_err(dk, fdk) <= cc.BWD_TOL
-    rdq, rdk = oracle.dense_bwd(da.double(), q.double(), k.double())
-    assert cf.rel_err(dq, rdq) > 0.5               # most differences are below 2^-64 here: far from the sign form
-    # no such range in float64 or in the generic float32 kernels
+    for where, value in (((0, 100, 3, 31), 1e-40), ((0, 5, 2, 7), float("inf"))):
+        print("case sign domain: one value", value, flush=True)
+        q, k = q0.clone(), k0.clone()
+        k[where] = value
+        dq, dk = _dense_bwd_gpu(q, k, da)
+        rdq, rdk = oracle.dense_bwd(da.double(), q.double(), k.double())
+        assert cf.rel_err(dq, rdq) <= cc.BWD_TOL and cf.rel_err(dk, rdk) <= cc.BWD_TOL, value
+    # float64 and the generic float32 kernels have no such range
     for e in (-70, 62):
         q, k = (q0 * 2.0 ** e).double(), (k0 * 2.0 ** e).double()
         dq, dk = _dense_bwd_gpu(q, k, da.double())
@@ -117,7 +113,7 @@ def test_sign_domain_of_the_fast_float32_backward():
         assert cf.rel_err(dq, rdq) <= 1e-12 and cf.rel_err(dk, rdk) <= 1e-12, e
         # fewer than 32 columns per token: the generic float32 kernels
         qn, kn, dan = q0[:, :, :2, :7].contiguous() * 2.0 ** e, k0[:, :, :2, :7].contiguous() * 2.0 ** e, da[..., :2].contiguous()
-        assert drv.lib().l1attn_dense_bwd_plan_info(B, T, 2, 7, info) == 0 and info[0] == 0
+        assert drv.lib().l1attn_dense_bwd_plan_info(B, T, 2, 7, info) == 0 and info[0] == 0 and info[15] == 0
         dq, dk = _dense_bwd_gpu(qn, kn, dan)
         rdq, rdk = oracle.dense_bwd(dan.double(), qn.double(), kn.double())
         assert cf.rel_err(dq, rdq) <= cc.BWD_TOL and cf.rel_err(dk, rdk) <= cc.BWD_TOL, e
