@@ -244,6 +244,11 @@ def set_dense_backward_form(loop_form=0, rank_sort=0):
     if rank_sort:
         _require_experimental("rank_merge", "the merge sort for the dense backward's column ranks")
     old, _dense_bwd_form = _dense_bwd_form, (int(loop_form), int(rank_sort))
+    if _dense_bwd_form != (0, 0) and _dense_bwd_form != old:
+        import warnings
+        warnings.warn("l1attn: the float32 dense backward now runs loop_form=%d, rank_sort=%d "
+                      "(l1attn_dense_bwd_ex_f32), kernels that have not passed their GPU tests yet" % _dense_bwd_form,
+                      RuntimeWarning, stacklevel=2)
     return old
 
 

@@ -726,6 +726,7 @@ def test_non_default_backward_forms_need_an_opt_in_by_name(monkeypatch):
         drv.set_dense_backward_form(loop_form=3)
     assert drv.set_dense_backward_form(0, 0) == (0, 0)
     drv.enable_experimental("bwd_pipe", "rank_merge")
-    assert drv.set_dense_backward_form(2, 1) == (0, 0) and drv._dense_bwd_form == (2, 1)
+    with pytest.warns(RuntimeWarning, match="loop_form=2, rank_sort=1"):   # said once per change, never silently
+        assert drv.set_dense_backward_form(2, 1) == (0, 0) and drv._dense_bwd_form == (2, 1)
     assert drv.dense_backward_plan(8, 4096, 16, 64)[14] == 2 and drv.dense_backward_plan(8, 4096, 16, 64, 0)[14] == 0
     assert drv.set_dense_backward_form() == (2, 1)
