@@ -136,3 +136,25 @@ def test_wip_sparse_half_gpu_tests_walk_on_stand_ins(cpu_stand_ins):
         t.test_half_empty_list(dt)
         for which in ("config4", "config5"):
             t.test_half_forward_benchmark_geometry(dt, which)
+
+
+def test_wip_backward_form_gpu_tests_walk_on_stand_ins(cpu_stand_ins, monkeypatch):
+    """tests/wip_bwd_prefetch_gpu.py (its smallest shape) and the backward test of tests/wip_rank_sort_gpu.py: the
+    plans they assert on come from the real library's host logic, the opt-in and the selection of the form run as
+    they will on the GPU, the backward itself is the CPU package's (whatever the form: all forms are specified to
+    give the same bits)."""
+    drv = cpu_stand_ins
+    monkeypatch.setattr(drv, "_dense_bwd_form", (0, 0))
+    t = _load("wip_bwd_prefetch_gpu")
+    monkeypatch.setattr(t, "DEV", "cpu")
+    assert [s for s, _ in t.SHAPES] == [(16, 1024, 8, 64), (4, 2048, 16, 64), (8, 4096, 16, 64)]
+    for shape, kind in t.SHAPES[1:]:  # the larger shapes: their plan assertions only
+        plans = [drv.dense_backward_plan(*shape, f) for f in (0, 1, 2)]
+        assert plans[0][3] == 1 and [p[14] for p in plans] == [0, 1, 2] and (plans[1][2], int(plans[1][9] > 1)) == kind
+    with pytest.warns(RuntimeWarning, match="loop_form"):
+        t.test_two_step_prefetch_equals_the_default_backward(*t.SHAPES[0])
+    assert drv._dense_bwd_form == (0, 0) and "bwd_pipe" in drv._enabled          # the form is put back afterwards
+    r = _load("wip_rank_sort_gpu")
+    with pytest.warns(RuntimeWarning, match="rank_sort=1"):
+        r.test_backward_on_merge_sort_ranks_equals_the_default_backward()
+    assert drv._dense_bwd_form == (0, 0) and "rank_merge" in drv._enabled

@@ -14,6 +14,7 @@ import torch
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda"
 
 # B, T, H, W and what bwd_plan makes of it: (rank, tiles per workgroup > 1)
 SHAPES = [((16, 1024, 8, 64), (0, 0)),     # second baseline configuration: sign form, one tile per workgroup
@@ -29,9 +30,9 @@ def test_two_step_prefetch_equals_the_default_backward(shape, kind):
     plans = [drv.dense_backward_plan(B, T, H, W, f) for f in (0, 1, 2)]
     assert plans[0][3] == 1 and [p[14] for p in plans] == [0, 1, 2]          # branch-free; the three forms
     assert (plans[1][2], int(plans[1][9] > 1)) == kind
-    g = torch.Generator(device="cuda").manual_seed(5)
-    q, k = (torch.randn(B, T, H, W, generator=g, device="cuda") for _ in range(2))
-    da = torch.empty(B, T, T, H, device="cuda")
+    g = torch.Generator(device=DEV).manual_seed(5)
+    q, k = (torch.randn(B, T, H, W, generator=g, device=DEV) for _ in range(2))
+    da = torch.empty(B, T, T, H, device=DEV)
     for b in range(B):
         da[b].normal_(generator=g)
     print("case backward with prefetch distance: one_step", shape, flush=True)
