@@ -76,8 +76,8 @@ int l1attn_dense_fwd_ws_f32(const float* q, const float* k, float* attn,
  * (cpp/l1attn_drv.cpp:7-11).  The f32 tiled path takes it as clamp(q*2^64 - k*2^64, -1, 1), which equals
  * sign(q-k) for every pair while all magnitudes are below 2^63 and all non-zero ones at least 2^-41;
  * a pre-pass over q and k checks exactly that on the device (a flag in the head of the workspace), and
- * when it does not hold -- tiny values, huge ones, infinities, NaN -- two more kernels of the same call
- * recompute dq and dk with comparisons.  The call stays asynchronous and the result is the reference's
+ * when it does not hold -- tiny values, huge ones, infinities, NaN -- one more kernel of the same call
+ * recomputes dq and dk with comparisons.  The call stays asynchronous and the result is the reference's
  * for every input; only the speed differs (O(T) reads per output element in the recomputation).
  * For 2048 <= T <= 8192 (and enough work to fill the GPU) sign() is taken from the column ranks of
  * l1attn_dense_column_ranks_f32 instead, exact for all finite inputs (no pre-pass, no flag); the
@@ -109,21 +109,26 @@ int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k,
                          int64_t B, int64_t T, int64_t H, int64_t W,
                          void* workspace, size_t workspace_bytes, void* stream);
 /*
- * l1attn_dense_bwd_f32 with its two internal choices as arguments; l1attn_dense_bwd_f32 is this call with
- * (0, 0).  The library reads no environment variable and keeps no state between calls: a caller that wants a
+ * l1attn_dense_bwd_f32 with its internal choices as arguments; l1attn_dense_bwd_f32 is this call with
+ * (0, 0, 0).  The library reads no environment variable and keeps no state between calls: a caller that wants a
  * non-default form says so here, per call.  Same workspace as l1attn_dense_bwd_f32.
  *   loop_form  step loop of the branch-free long-sequence plans: 0 one step of prefetch distance, 1 two steps,
  *              2 two steps with two LDS planes and one barrier per step.  Bit-identical results; other plans
  *              ignore it (l1attn_dense_bwd_plan_info_ex reports in info[14] what a shape runs).
  *   rank_sort  where the plan takes sign() from column ranks: 0 ranks from l1attn_dense_column_ranks_f32,
  *              1 from l1attn_dense_column_ranks_merge_f32.  Identical ranks.
- * Other values: L1ATTN_ERR_ARG.  No counterpart in the reference; the non-zero choices exist so that they can be
- * timed against the default and are not reached by the Python operators unless the caller opts in by name.
+ *   assume_sign_range  1: the caller vouches that every magnitude in q and k is below 2^63 and every non-zero
+ *              one at least 2^-41 (ordinary activations are); the range check and the fix-up launch of the tiled
+ *              path are left out, which saves one read of q and k -- about 20/T of the call, so it matters for
+ *              short sequences only.  Outside the vouched range the gradient follows clamp(q*2^64 - k*2^64, -1, 1)
+ *              in place of sign(q-k).  0: checked, exact for every input.
+ * Other values: L1ATTN_ERR_ARG.  No counterpart in the reference; the non-zero loop_form and rank_sort exist so that
+ * they can be timed against the default and are not reached by the Python operators unless the caller opts in by name.
  */
 int l1attn_dense_bwd_plan_info_ex(int64_t B, int64_t T, int64_t H, int64_t W, int loop_form, int64_t* info);
 int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk,
                             int64_t B, int64_t T, int64_t H, int64_t W, int loop_form, int rank_sort,
-                            void* workspace, size_t workspace_bytes, void* stream);
+                            int assume_sign_range, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Order-preserving integer ranks of q and k per column (b,h,w), the first stage of the f32

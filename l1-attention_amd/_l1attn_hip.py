@@ -82,7 +82,7 @@ def lib():
         L.l1attn_dense_bwd_plan_info_ex.restype = ctypes.c_int
         L.l1attn_dense_bwd_plan_info_ex.argtypes = [_c_i64] * 4 + [ctypes.c_int, _c_p]
         L.l1attn_dense_bwd_ex_f32.restype = ctypes.c_int
-        L.l1attn_dense_bwd_ex_f32.argtypes = [_c_p] * 5 + [_c_i64] * 4 + [ctypes.c_int] * 2 + [_c_p, _c_sz, _c_p]
+        L.l1attn_dense_bwd_ex_f32.argtypes = [_c_p] * 5 + [_c_i64] * 4 + [ctypes.c_int] * 3 + [_c_p, _c_sz, _c_p]
         for sfx in ("f32", "f64"):
             f = getattr(L, "l1attn_dense_fwd_" + sfx)
             f.restype = ctypes.c_int
@@ -229,6 +229,18 @@ def dense_forward_fixed(q, k):
 
 
 _dense_bwd_form = (0, 0)  # (loop_form, rank_sort) of l1attn_dense_bwd_ex_f32; (0, 0) is l1attn_dense_bwd_f32
+_assume_sign_range = False
+
+
+def assume_sign_range(flag=True):
+    """flag=True: from now on the caller vouches that q and k handed to the float32 dense backward hold magnitudes
+    below 2^63 and no non-zero magnitude below 2^-41 (ordinary activations do); the tiled backward then leaves out its
+    range check, which saves a read of q and k per call (about 20/T of the call: it matters below a few hundred
+    tokens).  Outside the vouched range sign(q-k) is replaced by clamp((q-k)*2^64, -1, 1).  Returns the previous
+    setting; the default, False, is exact for every input."""
+    global _assume_sign_range
+    old, _assume_sign_range = _assume_sign_range, bool(flag)
+    return old
 
 
 def set_dense_backward_form(loop_form=0, rank_sort=0):
@@ -278,9 +290,10 @@ def dense_backward(d_attn, q, k):
         ws_bytes = L.l1attn_dense_bwd_workspace_bytes(B, T, H, W) if sfx == "f32" else 0
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
         wsp = ptr(ws) if ws is not None else None
-        if sfx == "f32" and _dense_bwd_form != (0, 0):
+        if sfx == "f32" and (_dense_bwd_form != (0, 0) or _assume_sign_range):
             rc = L.l1attn_dense_bwd_ex_f32(ptr(d_attn), ptr(q), ptr(k), ptr(dq), ptr(dk), B, T, H, W,
-                                           _dense_bwd_form[0], _dense_bwd_form[1], wsp, ws_bytes, stream_of(q))
+                                           _dense_bwd_form[0], _dense_bwd_form[1], int(_assume_sign_range),
+                                           wsp, ws_bytes, stream_of(q))
         else:
             rc = getattr(L, "l1attn_dense_bwd_" + sfx)(
                 ptr(d_attn), ptr(q), ptr(k), ptr(dq), ptr(dk), B, T, H, W, wsp, ws_bytes, stream_of(q))

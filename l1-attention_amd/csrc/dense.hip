@@ -133,8 +133,8 @@ __global__ __launch_bounds__(256) void dense_bwd_generic_dk(const T* __restrict_
 // column ranks): clamp(q*2^64 - k*2^64, -1, 1) equals sign(q - k) for every pair when all magnitudes are below
 // 2^63 (no overflow) and every non-zero value is at least 2^-41 in magnitude (then all values, and so all their
 // differences, are whole multiples of 2^-64).  dense_bwd_sign_domain sets *flag when some value of q or k is
-// outside that (NaN and infinities included); the two kernels after it then recompute dq and dk with exact
-// comparisons, as the generic kernels do, and return at once when the flag is clear.  The flag lives in the
+// outside that (NaN and infinities included); the kernel after it then recomputes dq and dk with exact
+// comparisons, as the generic kernels do, and returns at once when the flag is clear.  The flag lives in the
 // caller's workspace and must be zero before dense_bwd_sign_domain runs.
 // ------------------------------------------------------------------------------------------
 
@@ -160,28 +160,29 @@ __global__ __launch_bounds__(256) void dense_bwd_sign_domain(const float* __rest
 	if (threadIdx.x == 0 && any_outside) atomicOr(flag, 1);
 }
 
-// DK false: one thread per dq element, src tokens summed in ascending order; DK true: one thread per dk element,
-// dst tokens in ascending order.  The arithmetic of dense_bwd_generic_dq / _dk.
-template <bool DK>
+// blockIdx.y == 0: one thread per dq element, src tokens summed in ascending order; blockIdx.y == 1: one thread per
+// dk element, dst tokens in ascending order.  The arithmetic of dense_bwd_generic_dq / _dk.
 __global__ __launch_bounds__(256) void dense_bwd_exact_if_flagged(const float* __restrict__ dA, const float* __restrict__ q,
-                                                                    const float* __restrict__ k, float* __restrict__ out,
-                                                                    int64_t B, int64_t Tn, int64_t H, int64_t W, float scale,
-                                                                    const int* __restrict__ flag)
+                                                                    const float* __restrict__ k, float* __restrict__ dq,
+                                                                    float* __restrict__ dk, int64_t B, int64_t Tn, int64_t H,
+                                                                    int64_t W, float scale, const int* __restrict__ flag)
 {
 	if (*flag == 0) return;
 	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
 	if (idx >= B * Tn * H * W) return;
+	const bool for_dk = blockIdx.y != 0;
 	const int64_t w = idx % W, h = (idx / W) % H, own = (idx / (W * H)) % Tn, b = idx / (W * H * Tn);
-	const float mine = DK ? k[idx] : q[idx];
+	const float mine = for_dk ? k[idx] : q[idx];
+	const float* const others = for_dk ? q : k;
 	float acc = 0;
 	for (int64_t o = 0; o < Tn; o++) {
-		const float other = (DK ? q : k)[((b * Tn + o) * H + h) * W + w];
-		const float ws = sgn_exact(DK ? other - mine : mine - other) * scale;
-		const int64_t s = DK ? own : o, t = DK ? o : own;
+		const float other = others[((b * Tn + o) * H + h) * W + w];
+		const float ws = sgn_exact(for_dk ? other - mine : mine - other) * scale;
+		const int64_t s = for_dk ? own : o, t = for_dk ? o : own;
 		const float g = dA[((b * Tn + s) * Tn + t) * H + h];
-		if (DK) acc -= ws * g; else acc += ws * g;
+		if (for_dk) acc -= ws * g; else acc += ws * g;
 	}
-	out[idx] = acc;
+	(for_dk ? dk : dq)[idx] = acc;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1358,11 +1359,15 @@ int l1attn_dense_bwd_plan_info(int64_t B, int64_t T, int64_t H, int64_t W, int64
 
 // rank_sort: 0 = column ranks from the library block radix sort (dense_rank.hip), 1 = from the merge sort of
 // rank_sort.hip; both give the same ranks
+// assume_sign_range: the caller vouches that every magnitude in q and k is below 2^63 and every non-zero one at
+// least 2^-41; the range check and the fix-up launch are then left out
 int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
-                            int64_t T, int64_t H, int64_t W, int loop_form, int rank_sort, void* workspace,
-                            size_t workspace_bytes, void* stream)
+                            int64_t T, int64_t H, int64_t W, int loop_form, int rank_sort, int assume_sign_range,
+                            void* workspace, size_t workspace_bytes, void* stream)
 {
-	if (!shape_ok(B, T, H, W) || loop_form < 0 || loop_form > 2 || rank_sort < 0 || rank_sort > 1) return L1ATTN_ERR_ARG;
+	if (!shape_ok(B, T, H, W) || loop_form < 0 || loop_form > 2 || rank_sort < 0 || rank_sort > 1 ||
+	    assume_sign_range < 0 || assume_sign_range > 1)
+		return L1ATTN_ERR_ARG;
 	const int64_t n = B * T * H * W;
 	if (n == 0) return L1ATTN_OK;
 	if (!d_attn || !q || !k || !dq || !dk) return L1ATTN_ERR_ARG;
@@ -1376,23 +1381,22 @@ int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k,
 	// Without column ranks the sign comes from the scaled difference: find out (on the device, without waiting)
 	// whether q and k are inside the range where that is exact; the fix-up launches at the end redo dq and dk
 	// with comparisons when they are not.
-	int* const flag = p.flag_bytes ? (int*)workspace : nullptr;
+	int* const flag = (p.flag_bytes && !assume_sign_range) ? (int*)workspace : nullptr;
+	if (p.flag_bytes) {
+		workspace = (char*)workspace + p.flag_bytes;
+		workspace_bytes -= p.flag_bytes;
+	}
 	if (flag) {
 		hipLaunchKernelGGL(dense_bwd_clear_flag, dim3(1), dim3(64), 0, st, flag);
 		L1_LAUNCH_CHECK();
 		const dim3 dgrid((unsigned)std::min<int64_t>(l1_cdiv(n, 256 * 8), 4096));
 		hipLaunchKernelGGL(dense_bwd_sign_domain, dgrid, dim3(256), 0, st, q, k, n, flag);
 		L1_LAUNCH_CHECK();
-		workspace = (char*)workspace + p.flag_bytes;
-		workspace_bytes -= p.flag_bytes;
 	}
 	const auto fix_up = [&]() -> int {
 		if (!flag) return L1ATTN_OK;
-		const dim3 egrid((unsigned)l1_cdiv(n, 256));
-		hipLaunchKernelGGL(dense_bwd_exact_if_flagged<false>, egrid, dim3(256), 0, st, d_attn, q, k, dq, B, T, H, W, scale,
-		                   (const int*)flag);
-		L1_LAUNCH_CHECK();
-		hipLaunchKernelGGL(dense_bwd_exact_if_flagged<true>, egrid, dim3(256), 0, st, d_attn, q, k, dk, B, T, H, W, scale,
+		const dim3 egrid((unsigned)l1_cdiv(n, 256), 2);
+		hipLaunchKernelGGL(dense_bwd_exact_if_flagged, egrid, dim3(256), 0, st, d_attn, q, k, dq, dk, B, T, H, W, scale,
 		                   (const int*)flag);
 		L1_LAUNCH_CHECK();
 		return L1ATTN_OK;
@@ -1457,7 +1461,7 @@ int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k,
 int l1attn_dense_bwd_f32(const float* d_attn, const float* q, const float* k, float* dq, float* dk, int64_t B,
                          int64_t T, int64_t H, int64_t W, void* workspace, size_t workspace_bytes, void* stream)
 {
-	return l1attn_dense_bwd_ex_f32(d_attn, q, k, dq, dk, B, T, H, W, 0, 0, workspace, workspace_bytes, stream);
+	return l1attn_dense_bwd_ex_f32(d_attn, q, k, dq, dk, B, T, H, W, 0, 0, 0, workspace, workspace_bytes, stream);
 }
 
 int l1attn_dense_bwd_f64(const double* d_attn, const double* q, const double* k, double* dq, double* dk, int64_t B,

@@ -495,7 +495,15 @@ def test_driver_control_flow_without_a_gpu(monkeypatch):
     a, = drv.dense_forward_fixed(q, k)
     assert a.shape == (B, T, T, H) and _FakeLib.calls[-2:] == ["l1attn_dense_fwd_fixed_workspace_bytes", "l1attn_dense_fwd_fixed_f32"]
     dq, dk = drv.dense_backward(torch.zeros(B, T, T, H), q, k)
-    assert dq.shape == q.shape and dk.shape == k.shape
+    assert dq.shape == q.shape and dk.shape == k.shape and _FakeLib.calls[-1] == "l1attn_dense_bwd_f32"
+    # a caller that vouches for the sign range, or selects a non-default form, goes through the _ex entry point
+    # (its argument list is checked against the header by the stand-in library)
+    monkeypatch.setattr(drv, "_assume_sign_range", False)
+    assert drv.assume_sign_range() is False
+    drv.dense_backward(torch.zeros(B, T, T, H), q, k)
+    assert _FakeLib.calls[-1] == "l1attn_dense_bwd_ex_f32" and drv.assume_sign_range(False) is True
+    drv.dense_backward(torch.zeros(B, T, T, H).double(), q.double(), k.double())
+    assert _FakeLib.calls[-1] == "l1attn_dense_bwd_f64"
     with pytest.raises(RuntimeError, match="d_attn must be"):
         drv.dense_backward(torch.zeros(B, T, T, H + 1), q, k)
     with pytest.raises(RuntimeError, match="one shape"):

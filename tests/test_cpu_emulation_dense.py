@@ -125,10 +125,10 @@ def test_dense_float64_and_ties(runner, tmp_path):
 def test_sign_domain_guard_of_the_tiled_backward(runner, tmp_path):
     """The tiled float32 backward without column ranks takes sign(q - k) from the difference of q * 2^64 and
     k * 2^64, which is exact while every magnitude is below 2^63 and every non-zero one at least 2^-41.  A pre-pass
-    raises a flag in the workspace otherwise and two fix-up kernels redo dq and dk with comparisons, so the result is
+    raises a flag in the workspace otherwise and a fix-up kernel redoes dq and dk with comparisons, so the result is
     the reference's sign() (cpp/l1attn_drv.cpp:7-11) for every input: tiny values whose differences the scaling
     would leave fractional, magnitudes it would overflow, infinities.  Inside the range the flag stays clear and
-    the fix-up kernels leave the tiled result alone."""
+    the fix-up kernel leaves the tiled result alone."""
     shape = (2, 64, 4, 32)                                                    # 32-token tiles, two per sequence
     g = torch.Generator().manual_seed(31)
     q0, k0 = (torch.randn(*shape, generator=g) for _ in range(2))
@@ -151,6 +151,19 @@ def test_sign_domain_guard_of_the_tiled_backward(runner, tmp_path):
     q = q0.clone()
     q[:, ::3] = 0.0
     assert _run(runner, tmp_path, shape, inputs=(q, k0, dA))["domain_flag"] == 0
+    # a caller that vouches for the range skips check and fix-up: same result inside the range (the flag word is
+    # never written), the stated formula -- not the sign -- outside it
+    inside = _run(runner, tmp_path, shape, inputs=(q0, k0, dA))
+    vouched = _run(runner, tmp_path, shape, inputs=(q0, k0, dA), extra=("assume",))
+    assert vouched["domain_flag"] == int.from_bytes(b"\xa5" * 4, "little", signed=True)
+    assert torch.equal(vouched["dq"], inside["dq"]) and torch.equal(vouched["dk"], inside["dk"])
+    tiny = _run(runner, tmp_path, shape, inputs=(q0 * 2.0 ** -70, k0 * 2.0 ** -70, dA), extra=("assume",))
+    s = ((tiny["q"].double() * 2.0 ** 64)[:, None] - (tiny["k"].double() * 2.0 ** 64)[:, :, None]).float().double().clamp(-1, 1)
+    sc = -1.0 / 32 ** 0.5
+    assert cf.rel_err(tiny["dq"], sc * torch.einsum("bsthw,bsth->bthw", s, dA.double())) <= 1e-4
+    assert cf.rel_err(tiny["dk"], -sc * torch.einsum("bsthw,bsth->bshw", s, dA.double())) <= 1e-4
+    rdq, _ = oracle.dense_bwd(dA.double(), tiny["q"].double(), tiny["k"].double())
+    assert cf.rel_err(tiny["dq"], rdq) > 0.5
     # plans that keep no flag: the untiled kernels compare exactly whatever the range
     r = _run(runner, tmp_path, (1, 12, 2, 7), scale=2.0 ** -70, seed=3)
     assert r["plan"]["tiled"] == 0 and r["domain_flag"] == -1
@@ -312,12 +325,11 @@ def test_launch_geometry_at_full_size(runner):
                             ("dense_bwd_reduce_dk<true, true, false>", (32768, 1, 1), 256, 0)]
     # without column ranks the backward brackets its kernels with the sign-domain check and the exact fix-up
     rcs, launches = _dims(runner, (16, 1024, 8, 64))
-    assert rcs["backward"] == "0" and [l[0] for l in launches[1:]][:7] == [
+    assert rcs["backward"] == "0" and [l[0] for l in launches[1:]][:6] == [
         "dense_bwd_clear_flag", "dense_bwd_sign_domain", "dense_bwd_f32_fast<64, 512, 4, false, false, true>",
-        "dense_bwd_reduce_dk<true, false, false>", "dense_bwd_exact_if_flagged<false>", "dense_bwd_exact_if_flagged<true>",
-        "fixed_absmax"]
+        "dense_bwd_reduce_dk<true, false, false>", "dense_bwd_exact_if_flagged", "fixed_absmax"]
     assert launches[3] == ("dense_bwd_f32_fast<64, 512, 4, false, false, true>", (16, 1, 16), 512, 8704)
-    assert launches[2][1] == (4096, 1, 1) and launches[5][1] == (16 * 1024 * 8 * 64 // 256, 1, 1)
+    assert launches[2][1] == (4096, 1, 1) and launches[5][1] == (16 * 1024 * 8 * 64 // 256, 2, 1)
     assert _dims(runner, (2, 64, 4, 32))[0]["backward"] == "0"
     kernels = set()
     for T in (16, 32, 64, 128, 256):
