@@ -363,6 +363,11 @@ def instruction_rates():
     return rates
 
 
+def _l1attn_hip_setting(name):
+    import _l1attn_hip
+    return getattr(_l1attn_hip, name)
+
+
 def reference_sweep(num_runs=10):
     """The reference's own timing grid (benchmark.py:57-66): B=512, H=8, T in {16,...,256}, W in
     {16,32,33,64,65,96,97,128}, forward and backward of L1AttnFn timed separately as averages over num_runs.
@@ -398,7 +403,8 @@ def reference_sweep(num_runs=10):
             N = B * T * T * H * W
             row = {"sweep": "benchmark.py:57-66", "batch_size": B, "seq_length": T, "n_heads": H, "width": W,
                    "avg_forward_ms": fwd_ms, "avg_backward_ms": bwd_ms,
-                   "fwd_tops": 2 * N / fwd_ms / 1e9, "bwd_tops": 4 * N / bwd_ms / 1e9}
+                   "fwd_tops": 2 * N / fwd_ms / 1e9, "bwd_tops": 4 * N / bwd_ms / 1e9,
+                   "sign_range_checked": not _l1attn_hip_setting("_assume_sign_range")}
             print(json.dumps(row), flush=True)
             rows.append(row)
             del q, k, dA, attn
@@ -574,6 +580,9 @@ def main():
                     help="A/B aid: step loop of the long-sequence dense backward (0 = the default entry point)")
     ap.add_argument("--rank-sort", choices=("radix", "merge"), default="radix",
                     help="A/B aid: sort behind the dense backward's column ranks (radix = the default entry point)")
+    ap.add_argument("--assume-sign-range", action="store_true",
+                    help="A/B aid: leave out the dense backward's sign-range check (the caller vouches for q and k); "
+                         "matters for the short sequences of --sweep")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: only run three 1 GiB device-to-device copies, the known-size "
                          "kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -589,6 +598,8 @@ def main():
         sys.exit(3)
     import _l1attn_hip
     _l1attn_hip.lib()  # fail here, loudly, if the HIP library is not built
+    if args.assume_sign_range:
+        _l1attn_hip.assume_sign_range(True)
     if args.bwd_form or args.rank_sort == "merge":
         _l1attn_hip.enable_experimental(*([("bwd_pipe")] if args.bwd_form else []),
                                         *([("rank_merge")] if args.rank_sort == "merge" else []))
