@@ -272,7 +272,7 @@ def isa_digests(asm_text, mask_kernarg_offsets=False):
             l = re.sub(r"^(s_load_dword\w* \S+ s\[%d:%d\],) \S+" % (karg[kern], karg[kern] + 1), r"\1 KERNARG_OFFSET", l)
             # the pair holds the argument pointer until the first instruction (in layout order) that names it as
             # its destination; what is loaded through it afterwards is not a kernel argument
-            m = re.match(r"(?!s_cmp|s_bitcmp|s_cbranch|s_store)\S+ (s\[\d+:\d+\]|s\d+)\b", l)
+            m = re.match(r"(?!s_cmp|s_bitcmp|s_cbranch)\S+ (s\[\d+:\d+\]|s\d+)\b", l)
             if m and _sregs(m.group(1)) & {karg[kern], karg[kern] + 1}:
                 overwritten.add(kern)
         streams.setdefault(kern, []).append(l)
