@@ -1376,13 +1376,15 @@ int l1attn_dense_bwd_ex_f32(const float* d_attn, const float* q, const float* k,
 	if (!p.fast) return launch_bwd_generic<float>(d_attn, q, k, dq, dk, B, T, H, W, st);
 	const float scale = (float)(-1.0 / sqrt((double)W));
 	const int64_t HW = H * W;
-	const size_t need = p.flag_bytes + p.per_batch_bytes;
-	if (need && (!workspace || workspace_bytes < need)) return L1ATTN_ERR_WORKSPACE;
+	// the head of the workspace belongs to the flag whether this call uses it or not, so that one layout serves
+	// every call on a shape; a vouched call on a plan without partial arrays needs no workspace at all
+	const bool uses_workspace = p.per_batch_bytes > 0 || (p.flag_bytes > 0 && !assume_sign_range);
+	if (uses_workspace && (!workspace || workspace_bytes < p.flag_bytes + p.per_batch_bytes)) return L1ATTN_ERR_WORKSPACE;
 	// Without column ranks the sign comes from the scaled difference: find out (on the device, without waiting)
-	// whether q and k are inside the range where that is exact; the fix-up launches at the end redo dq and dk
+	// whether q and k are inside the range where that is exact; the fix-up launch at the end redoes dq and dk
 	// with comparisons when they are not.
 	int* const flag = (p.flag_bytes && !assume_sign_range) ? (int*)workspace : nullptr;
-	if (p.flag_bytes) {
+	if (uses_workspace && p.flag_bytes) {
 		workspace = (char*)workspace + p.flag_bytes;
 		workspace_bytes -= p.flag_bytes;
 	}
