@@ -18,7 +18,10 @@
 #include <algorithm>
 #include <atomic>
 #include <barrier>
+#include <condition_variable>
+#include <functional>
 #include <memory>
+#include <mutex>
 #include <thread>
 #include <vector>
 
@@ -212,6 +215,69 @@ static inline void emu_buf_fadd(float x, __amdgpu_buffer_rsrc_t r, int v, int s)
 // every thread of the workgroup must reach it (a thread that has returned would hang the others, as it may on a GPU)
 static inline void __syncthreads() { emu::wg_barrier->arrive_and_wait(); }
 
+namespace emu {
+// The OS threads that play the GPU threads, kept from launch to launch (a library call is dozens of launches):
+// run(nt, f) has threads 0..nt-1 execute f(thread number) and returns when all have finished.
+class Pool {
+	std::vector<std::thread> threads_;
+	std::mutex m_;
+	std::condition_variable start_, done_;
+	std::function<void(unsigned)> job_;
+	unsigned active_ = 0, finished_ = 0;
+	long generation_ = 0;
+	bool stop_ = false;
+	void loop(unsigned id)
+	{
+		long seen = 0;
+		for (;;) {
+			std::function<void(unsigned)> job;
+			{
+				std::unique_lock<std::mutex> lk(m_);
+				start_.wait(lk, [&] { return stop_ || generation_ != seen; });
+				if (stop_) return;
+				seen = generation_;
+				if (id >= active_) continue;
+				job = job_;
+			}
+			job(id);
+			std::lock_guard<std::mutex> lk(m_);
+			if (++finished_ == active_) done_.notify_all();
+		}
+	}
+
+public:
+	void run(unsigned nt, std::function<void(unsigned)> f)
+	{
+		std::unique_lock<std::mutex> lk(m_);
+		// a new thread starts with seen = 0 and generation_ >= 1 below, so it picks this job up
+		while (threads_.size() < nt) {
+			const unsigned id = (unsigned)threads_.size();
+			threads_.emplace_back([this, id] { loop(id); });
+		}
+		job_ = std::move(f);
+		active_ = nt;
+		finished_ = 0;
+		generation_++;
+		start_.notify_all();
+		done_.wait(lk, [&] { return finished_ == active_; });
+	}
+	~Pool()
+	{
+		{
+			std::lock_guard<std::mutex> lk(m_);
+			stop_ = true;
+		}
+		start_.notify_all();
+		for (auto& t : threads_) t.join();
+	}
+};
+inline Pool& pool()
+{
+	static Pool p;
+	return p;
+}
+}
+
 template <typename K, typename... A>
 static inline void emu_launch(const char* name, K kernel, dim3 grid, dim3 block, size_t lds, A... args)
 {
@@ -250,9 +316,7 @@ static inline void emu_launch(const char* name, K kernel, dim3 grid, dim3 block,
 			step.arrive_and_wait();
 		}
 	};
-	std::vector<std::thread> pool;
-	for (unsigned t = 0; t < nt; t++) pool.emplace_back(worker, t);
-	for (auto& th : pool) th.join();
+	emu::pool().run(nt, worker);  // the OS threads are kept from launch to launch
 	emu::n_threads_run += (long)nt * nblocks;
 }
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
