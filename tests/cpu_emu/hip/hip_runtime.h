@@ -73,7 +73,12 @@ inline std::unique_ptr<std::barrier<>> wg_barrier;  // the running workgroup's _
 // Lanes of a wavefront run in lockstep on the GPU; here they are OS threads, so every cross-lane exchange is
 // bracketed by a barrier among the wave's 64 threads.
 inline std::vector<std::unique_ptr<std::barrier<>>> wave_barrier;
-inline std::vector<double> wave_slots;  // 64 exchange slots per wave
+// 64 exchange slots per wave, in two planes that successive exchanges alternate between: a lane that is already
+// writing its value for exchange n+1 cannot disturb a lane still reading exchange n, so one barrier per exchange is
+// enough (a lane reaches exchange n+2, which reuses the plane of n, only after every lane has arrived at the barrier
+// of n+1, hence finished reading n).  All lanes of a wave take part in every exchange, so their counts agree.
+inline std::vector<double> wave_slots[2];
+inline thread_local unsigned exchange_count = 0;  // reset at the start of every workgroup
 // A runner may ask to see every launch (kernel expression as written at the launch site, grid, block, dynamic LDS
 // bytes) and may set `dry`: the launch is then reported and checked against the limits of a HIP launch, not run.
 inline void (*on_launch)(const char* kernel, dim3 grid, dim3 block, size_t lds) = nullptr;
@@ -81,6 +86,14 @@ inline bool dry = false;
 inline unsigned char* dynamic_lds = nullptr;  // the launch's dynamically sized LDS array, exactly `lds` bytes
 inline unsigned flat_tid() { return threadIdx_.x + blockDim_.x * (threadIdx_.y + blockDim_.y * threadIdx_.z); }
 inline void wave_sync() { wave_barrier[flat_tid() >> 6]->arrive_and_wait(); }
+// one cross-lane exchange: publish x, wait for the wave, return the plane to read the other lanes' values from
+inline const std::vector<double>& exchange(double x)
+{
+	std::vector<double>& plane = wave_slots[exchange_count++ & 1u];
+	plane[flat_tid()] = x;
+	wave_sync();
+	return plane;
+}
 // Barrier among a subset of a wave's lanes, keyed by the subset's lowest lane (disjoint subsets of one wave may
 // wait at the same time): the last lane to arrive opens the gate for the others.
 struct LaneGate { std::atomic<int> count{0}, generation{0}; };
@@ -124,11 +137,7 @@ template <typename T>
 static inline T __shfl_xor(T x, int lane_mask)
 {
 	const unsigned tid = emu::flat_tid(), base = tid & ~63u;
-	emu::wave_slots[tid] = (double)x;
-	emu::wave_sync();
-	const T r = (T)emu::wave_slots[base + ((tid ^ (unsigned)lane_mask) & 63u)];
-	emu::wave_sync();
-	return r;
+	return (T)emu::exchange((double)x)[base + ((tid ^ (unsigned)lane_mask) & 63u)];
 }
 template <typename T>
 static inline T __shfl_xor(T x, int lane_mask, int width)
@@ -142,23 +151,18 @@ static inline T __shfl_up(T x, unsigned delta, int width)
 {
 	if (width != 64) abort();
 	const unsigned tid = emu::flat_tid();
-	emu::wave_slots[tid] = (double)x;
-	emu::wave_sync();
-	const T r = (tid & 63u) >= delta ? (T)emu::wave_slots[tid - delta] : x;
-	emu::wave_sync();
-	return r;
+	const std::vector<double>& plane = emu::exchange((double)x);
+	return (tid & 63u) >= delta ? (T)plane[tid - delta] : x;
 }
 // bit l = predicate of lane l.  Every lane of the wave must call it (the emulated waves are always full or end
 // with the workgroup: a lane beyond it reads as 0).
 static inline unsigned long long __ballot(int pred)
 {
 	const unsigned tid = emu::flat_tid(), base = tid & ~63u;
-	emu::wave_slots[tid] = pred ? 1.0 : 0.0;
-	emu::wave_sync();
+	const std::vector<double>& plane = emu::exchange(pred ? 1.0 : 0.0);
 	unsigned long long m = 0;
-	for (unsigned l = 0; l < 64 && base + l < emu::wave_slots.size(); l++)
-		if (emu::wave_slots[base + l] != 0.0) m |= 1ull << l;
-	emu::wave_sync();
+	for (unsigned l = 0; l < 64 && base + l < plane.size(); l++)
+		if (plane[base + l] != 0.0) m |= 1ull << l;
 	return m;
 }
 static inline int __popcll(unsigned long long x) { return __builtin_popcountll(x); }
@@ -176,11 +180,8 @@ static inline int atomicMax(int* p, int v)
 static inline int emu_dpp_row_shr(int src, int ctrl)
 {
 	const unsigned tid = emu::flat_tid(), n = (unsigned)ctrl & 15u;
-	emu::wave_slots[tid] = (double)src;
-	emu::wave_sync();
-	const int r = ((tid & 15u) >= n) ? (int)emu::wave_slots[tid - n] : 0;
-	emu::wave_sync();
-	return r;
+	const std::vector<double>& plane = emu::exchange((double)src);
+	return ((tid & 15u) >= n) ? (int)plane[tid - n] : 0;
 }
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound_ctrl) \
 	(static_cast<void>(sizeof(char[((ctrl) > 0x110 && (ctrl) < 0x120 && (bound_ctrl)) ? 1 : -1])), emu_dpp_row_shr(src, ctrl))
@@ -308,9 +309,11 @@ static inline void emu_launch(const char* name, K kernel, dim3 grid, dim3 block,
 				emu::wave_barrier.clear();
 				for (unsigned w = 0; w < (nt + 63) / 64; w++)
 					emu::wave_barrier.emplace_back(new std::barrier<>(std::min(64u, nt - w * 64)));
-				emu::wave_slots.assign((nt + 63) / 64 * 64, 0.0);
+				emu::wave_slots[0].assign((nt + 63) / 64 * 64, 0.0);
+				emu::wave_slots[1].assign((nt + 63) / 64 * 64, 0.0);
 				emu::lane_gates.reset(new emu::LaneGate[(nt + 63) / 64 * 64]);
 			}
+			emu::exchange_count = 0;
 			step.arrive_and_wait();
 			kernel(args...);
 			step.arrive_and_wait();
