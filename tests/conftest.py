@@ -33,7 +33,8 @@ RUNNERS = {"fused": ("fused", "g++", "address,undefined"), "sparse": ("sparse", 
            "ranks": ("ranks", "g++", "address,undefined"), "dense": ("dense", "g++", "address,undefined"),
            "fused_tsan": ("fused", "g++", "thread"), "sparse_tsan": ("sparse", CLANG, "thread"),
            "dense_tsan": ("dense", "g++", "thread"), "ranks_tsan": ("ranks", "g++", "thread"),
-           "coo": ("coo", "g++", "address,undefined"), "coo_tsan": ("coo", "g++", "thread")}
+           "coo": ("coo", "g++", "address,undefined"), "coo_tsan": ("coo", "g++", "thread"),
+           "ranks_lib": ("ranks_lib", "g++", "address,undefined"), "ranks_lib_tsan": ("ranks_lib", "g++", "thread")}
 
 
 @pytest.fixture(scope="session")
@@ -112,3 +113,13 @@ def emu_coo(_emu_builds):
 @pytest.fixture(scope="session")
 def emu_coo_tsan(_emu_builds):
     return _emu_runner(_emu_builds, "coo_tsan")
+
+
+@pytest.fixture(scope="session")
+def emu_ranks_lib(_emu_builds):
+    return _emu_runner(_emu_builds, "ranks_lib")
+
+
+@pytest.fixture(scope="session")
+def emu_ranks_lib_tsan(_emu_builds):
+    return _emu_runner(_emu_builds, "ranks_lib_tsan")

@@ -235,9 +235,11 @@ def test_fixed_point_prepass_kernels_on_cpu(tmp_path):
     assert np.all(uq[1, :, 2] == 2 ** 31) and np.all(uk[1, :, 2] == 2 ** 31)
 
 
-@pytest.fixture(scope="module")
-def ranks_runner(emu_ranks):
-    return emu_ranks
+@pytest.fixture(scope="module", params=["merge", "library"])
+def ranks_runner(request):
+    """The rank kernel written for this library (csrc/rank_sort.hip), and the one the backward uses by default
+    (csrc/dense_rank.hip) with a host stand-in for the library block sort it calls: same ranks by definition."""
+    return request.getfixturevalue("emu_ranks" if request.param == "merge" else "emu_ranks_lib")
 
 
 def _reference_ranks(q, k):
@@ -260,8 +262,9 @@ def _reference_ranks(q, k):
 
 @pytest.mark.parametrize("shape", [(1, 4096, 1, 2), (1, 1000, 2, 2), (2, 300, 1, 3), (1, 2049, 1, 2), (1, 5000, 1, 1),
                                    (1, 1, 1, 5), (1, 513, 3, 1)])
-def test_merge_sort_column_ranks_on_cpu(tmp_path, shape, ranks_runner):
-    """The merge-sort rank kernel (csrc/rank_sort.hip; registers, LDS and barriers only) under AddressSanitizer:
+def test_column_rank_kernels_on_cpu(tmp_path, shape, ranks_runner):
+    """Both column-rank kernels (csrc/rank_sort.hip: registers, LDS and barriers only; csrc/dense_rank.hip around
+    a stand-in for the library sort) under AddressSanitizer:
     every items-per-thread instantiation (T up to 512, 1024, 2048, 4096, 8192), ragged lengths (padding keys),
     planted ties between q and k, repeated k values, both zeros; ranks equal their definition exactly, and
     clamp(rq - rk, 0, 1) is 1, 1/2, 0 for q >, ==, < k on every pair of a column."""
@@ -297,10 +300,13 @@ def test_merge_sort_column_ranks_on_cpu(tmp_path, shape, ranks_runner):
         assert np.array_equal(2 * hv - 1, sign)
 
 
-@pytest.mark.parametrize("shape", [(1, 1000, 1, 2), (1, 2049, 1, 1)])
-def test_merge_sort_column_ranks_have_no_data_race(tmp_path, shape, emu_ranks_tsan):
+@pytest.mark.parametrize("shape,kernel", [((1, 1000, 1, 2), "merge"), ((1, 2049, 1, 1), "merge"),
+                                          ((2, 700, 1, 3), "library")])
+def test_column_rank_kernels_have_no_data_race(tmp_path, shape, kernel, request):
     """The merge rounds work in place in LDS: every thread reads its inputs, a barrier, every thread writes its
-    outputs, a barrier.  Under ThreadSanitizer a thread that wrote before another had read would be a data race."""
+    outputs, a barrier.  Under ThreadSanitizer a thread that wrote before another had read would be a data race.
+    The default kernel hands its sorted keys to every thread's searches through LDS behind one barrier."""
+    emu_ranks_tsan = request.getfixturevalue("emu_ranks_tsan" if kernel == "merge" else "emu_ranks_lib_tsan")
     B, T, H, W = shape
     g = torch.Generator().manual_seed(sum(shape))
     q, k = (torch.randn(B, T, H, W, generator=g) for _ in range(2))

@@ -1,7 +1,8 @@
 """CPU-only: the GPU test files run end to end on the CPU -- the real Python operators and drivers, the real ctypes
 binding with its argtypes, and a library built from the product's kernel sources for the host
-(tests/cpu_emu/lib_*.cpp: dense.hip, fixed.hip, fused.hip, rank_sort.hip and sparse.hip as they are, GPU threads as OS
-threads; host stand-ins only for coo.hip and the library sort, whose kernels cannot run that way).
+(tests/cpu_emu/lib_*.cpp: dense.hip, dense_rank.hip, fixed.hip, fused.hip, rank_sort.hip and sparse.hip as they are,
+GPU threads as OS threads; host stand-ins only for the library block sort inside dense_rank.hip and, to keep the runs
+short, for coo.hip, whose kernels run from source in tests/test_cpu_emulation_coo.py).
 
 Everything else on the CPU either runs the kernels through C++ runners (which call the entry points themselves) or
 walks the drivers against stand-ins that accept anything.  Neither notices a driver that passes the right kinds of
@@ -21,8 +22,8 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 EMU = os.path.join(HERE, "cpu_emu")
 CLANG = "/opt/rocm/llvm/bin/clang++"
-PARTS = (("lib_dense", "g++"), ("lib_fixed", "g++"), ("lib_fused", "g++"), ("lib_ranks", "g++"), ("lib_sparse", CLANG),
-         ("lib_host", "g++"))
+PARTS = (("lib_dense", "g++"), ("lib_fixed", "g++"), ("lib_fused", "g++"), ("lib_ranks", "g++"),
+         ("lib_ranks_default", "g++"), ("lib_sparse", CLANG), ("lib_host", "g++"))
 
 pytestmark = pytest.mark.skipif(not os.path.exists(CLANG), reason="needs ROCm's clang++ (bfloat16 and float16 on the host)")
 

@@ -4,7 +4,7 @@ l1attn_dense_bwd_ex_f32(rank_sort=1) must equal the default backward bit for bit
 
 This file has not run on a GPU yet, which is why its name keeps it out of pytest's collection
 (run it as `python -m pytest tests/wip_rank_sort_gpu.py -m gpu`); rename it to test_*.py once it has passed there.
-The kernel itself runs on the CPU in tests/test_cpu_emulation.py::test_merge_sort_column_ranks_on_cpu.
+The kernel itself runs on the CPU in tests/test_cpu_emulation.py::test_column_rank_kernels_on_cpu.
 """
 import os
 
